@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused P-partial reduce + residual-add + RMSNorm path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--sweep]
+
+A step is one call of the fused op (one kernel launch) on one batch of synthetic
+input that is already resident in HBM.  The default workload is the headline
+configuration: one rank's shard of a Llama-70B TP=8 layer, P=8 partials of
+[256, 8192] bf16 (a T=2048 batch).  Consecutive steps use different input sets
+(rotation over more than 1 GiB) so that no step finds its operands in the 256 MB
+last-level cache.  Prints ONE JSON line on stdout; progress goes to stderr.
+
+Fields beyond the usual ones:
+  roofline      HBM roofline of the norm kernel: algorithmic bytes per launch
+                divided by the mean launch duration measured with HIP events around
+                every launch of the timed region (same stream as the kernel).
+  cpu_baseline  the CPU checker (oracle/, a port of the reference's
+                csrc/cpu/layernorm.cpp extended to P partials) timed on this box's
+                host cores on the same workload, for context only.
+  sweep         (--sweep) µs/call and GB/s of every benchmark configuration, and the
+                weave configuration's overlap figures.
+"""
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+ROTATION_BYTES = (1 << 30) + (1 << 28) # > 1 GiB of distinct operands before any reuse
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default="c2_llama70b_tp8_shard@T256")
+    ap.add_argument("--max-ctas", type=int, default=0, help="grid cap (0 = library default)")
+    ap.add_argument("--sweep", action="store_true", help="also time every configuration")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline")
+    return ap.parse_args()
+
+
+class NormRunner:
+    """Pre-binds the C-ABI call for each input set so the timed loop is one ctypes
+    call per step (argument checks were done once, here, by the regular shim)."""
+
+    def __init__(self, cfg, nsets, max_ctas, device):
+        import torch
+        from tokenweave_amd import _custom_ops as ops
+        from tokenweave_amd import _lib
+        from tokenweave_amd import workloads as wl
+        self.cfg, self.torch, self.lib = cfg, torch, _lib.lib()
+        self.sets, self.calls = [], []
+        for i in range(nsets):
+            inp = wl.make_norm_inputs(cfg, device, seed_offset=i)
+            out = inp.partials[0]  # y lands on this rank's staging rows (rank 0)
+            # one checked call through the public shim validates the arguments
+            ops.reduce_add_rms_norm(inp.partials, out, inp.residual, inp.weight, cfg.eps,
+                                    max_ctas or None)
+            ptrs = (ctypes.c_void_p * cfg.P)(*[p.data_ptr() for p in inp.partials])
+            self.sets.append((inp, ptrs))
+            self.calls.append((ptrs, cfg.P, out.data_ptr(), inp.residual.data_ptr(),
+                               inp.weight.data_ptr(), cfg.T, cfg.H, max_ctas, cfg.eps))
+        torch.cuda.synchronize()
+        self.fn = self.lib.tw_reduce_add_rms_norm
+
+    def step(self, i, stream_ptr):
+        rc = self.fn(*self.calls[i % len(self.calls)], stream_ptr)
+        if rc != 0:
+            raise RuntimeError(self.lib.tw_last_error().decode())
+
+
+def time_norm(cfg, steps, warmup, max_ctas, device, per_launch_events=True):
+    """Returns dict(ms_per_step, gbps, kernel_us_mean, kernel_us_median)."""
+    import torch
+    nsets = max(2, min(64, -(-ROTATION_BYTES // cfg.bytes)))
+    free, _ = torch.cuda.mem_get_info()
+    set_bytes = (cfg.P + 1) * cfg.T * cfg.H * 2 + cfg.H * 2
+    nsets = max(2, min(nsets, int(free * 0.6) // (set_bytes * 3)))  # fp32 staging while generating
+    runner = NormRunner(cfg, nsets, max_ctas, device)
+    stream = torch.cuda.current_stream()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    for i in range(warmup):
+        runner.step(i, sp)
+    torch.cuda.synchronize()
+    # timed region: exactly `steps` launches between two synchronisation points
+    t0 = time.perf_counter()
+    for i in range(steps):
+        runner.step(i, sp)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    res = {"ms_per_step": wall * 1e3 / steps, "gbps": cfg.bytes * steps / wall / 1e9,
+           "nsets": nsets}
+    if per_launch_events:
+        n = min(steps, 200)
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+        stops = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+        for i in range(n):
+            starts[i].record(stream)
+            runner.step(i, sp)
+            stops[i].record(stream)
+        torch.cuda.synchronize()
+        us = [s.elapsed_time(e) * 1e3 for s, e in zip(starts, stops)]
+        res["kernel_us_mean"] = statistics.fmean(us)
+        res["kernel_us_median"] = statistics.median(us)
+        res["kernel_us_min"] = min(us)
+    del runner
+    torch.cuda.empty_cache()
+    return res
+
+
+def cpu_baseline(cfg, budget_s):
+    """Times the CPU checker on a bounded sample of the workload: the same shapes,
+    rows capped so one call stays around a second, repeated inside the budget."""
+    import numpy as np
+    import torch
+    from oracle import tw_oracle as O
+    from tokenweave_amd import workloads as wl
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    rows = min(cfg.T, 1024)
+    sample = cfg.with_tokens(rows)
+    inp = wl.make_norm_inputs(sample, "cpu")
+    bits = lambda t: np.ascontiguousarray(t.contiguous().view(torch.int16).numpy().view(np.uint16))
+    parts = [bits(p) for p in inp.partials]
+    r, w = bits(inp.residual), bits(inp.weight)
+    y = np.empty_like(r)
+    O.reduce_add_rms_norm(parts, r, w, cfg.eps, y=y)  # warm-up (page faults, thread pool)
+    times, t_end = [], time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 200):
+        t0 = time.perf_counter()
+        O.reduce_add_rms_norm(parts, r, w, cfg.eps, y=y)
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    return {"value": round(sample.bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads,
+            "kind": "port",
+            "sample": f"{len(times)} calls of P={sample.P} T={rows} H={sample.H} "
+                      f"({sample.bytes} algorithmic bytes each), median {med * 1e6:.0f} us/call, "
+                      f"OpenMP over rows with {threads} threads"}
+
+
+def time_weave(device, norm_cap, gemm_cap, iters=30):
+    """Config 5: GEMM of the 2458-row split on the current stream, fused norm of the
+    1638-row split on a second stream.  Returns serial / overlapped times."""
+    import torch
+    import tokenweave_amd as tw
+    from tokenweave_amd import _custom_ops as ops
+    from tokenweave_amd import workloads as wl
+    cfg = wl.C5_NORM
+    inp = wl.make_norm_inputs(cfg, device)
+    g = wl.make_gemm_inputs(device=device)
+    Ta = g.a.shape[0]
+    stage = torch.zeros((Ta, cfg.H), dtype=torch.bfloat16, device=device)
+    side = torch.cuda.Stream()
+
+    def gemm():
+        ops.gemm_bf16_nt(stage, g.a, g.b, max_cus=gemm_cap or None)
+
+    def norm():
+        ops.reduce_add_rms_norm(inp.partials, inp.partials[0], inp.residual, inp.weight, cfg.eps,
+                                norm_cap or None)
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(iters):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            ts.append(a.elapsed_time(b) * 1e3)
+        return statistics.median(ts)
+
+    t_a, t_b = timed(gemm), timed(norm)
+    t_ser = timed(lambda: (gemm(), norm()))
+    t_ovl = timed(lambda: tw.weave_norm_gemm(gemm, norm, side))
+    flops = 2.0 * Ta * cfg.H * g.a.shape[1]
+    return {"gemm_us": t_a, "norm_us": t_b, "serial_us": t_ser, "overlap_us": t_ovl,
+            "speedup": t_ser / t_ovl, "overlap_eff": (t_ser - t_ovl) / min(t_a, t_b),
+            "gemm_tflops_alone": flops / t_a / 1e6,
+            "gemm_mfma_util_alone": flops / t_a / 1e6 / MFMA_BF16_PEAK_TFLOPS,
+            "norm_gbps_alone": cfg.bytes / t_b / 1e3, "norm_cap": norm_cap, "gemm_cap": gemm_cap}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one rank's work on ONE GPU; --gpus must be 1 "
+                 "(this path has no collectives to scale across GPUs)")
+    import torch
+    from tokenweave_amd import workloads as wl
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    device = "cuda:0"
+    torch.cuda.set_device(0)
+    cfgs = wl.norm_configs()
+    if args.workload not in cfgs:
+        sys.exit(f"unknown workload {args.workload}; choose from {sorted(cfgs)}")
+    cfg = cfgs[args.workload]
+    log(f"[bench] {torch.cuda.get_device_name(0)}; workload {cfg.name}: P={cfg.P} T={cfg.T} "
+        f"H={cfg.H} bytes/call={cfg.bytes}")
+
+    res = time_norm(cfg, args.steps, args.warmup, args.max_ctas, device)
+    log(f"[bench] {res}")
+    kernel_us = res["kernel_us_mean"]
+    achieved = cfg.bytes / kernel_us / 1e3
+    out = {
+        "metric": "fused P-partial reduce+add+RMSNorm GB/s (% HBM peak), us/call, H=8192",
+        "value": round(res["gbps"], 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(res["ms_per_step"], 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": cfg.name, "P": cfg.P, "T": cfg.T, "H": cfg.H, "eps": cfg.eps,
+                   "bytes_per_call": cfg.bytes, "rotating_input_sets": res["nsets"],
+                   "max_ctas": args.max_ctas},
+        "pct_hbm_peak": round(100.0 * res["gbps"] / HBM_PEAK_GBPS, 2),
+        "us_per_call": round(res["ms_per_step"] * 1e3, 3),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "row_norm_bf16_kernel<8,1,true,false>",
+                     "kernel_us_mean": round(kernel_us, 3),
+                     "kernel_us_median": round(res["kernel_us_median"], 3)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
+        log(f"[bench] cpu_baseline {out['cpu_baseline']}")
+    if args.sweep:
+        sweep = {}
+        for name, c in cfgs.items():
+            steps = max(20, min(args.steps, int(2e9 // c.bytes)))
+            r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device)
+            sweep[name] = {"P": c.P, "T": c.T, "H": c.H, "bytes": c.bytes,
+                           "us_per_call": round(r["ms_per_step"] * 1e3, 3),
+                           "kernel_us": round(r["kernel_us_mean"], 3),
+                           "gbps": round(c.bytes / r["kernel_us_mean"] / 1e3, 1),
+                           "pct_hbm_peak": round(c.bytes / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
+            log(f"[sweep] {name}: {sweep[name]}")
+        w = time_weave(device, norm_cap=64, gemm_cap=0)
+        sweep["c5_weave"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}
+        log(f"[sweep] c5_weave: {sweep['c5_weave']}")
+        out["sweep"] = sweep
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,149 @@
+/*
+ * tokenweave_amd — C ABI of the MI355X (gfx950) fused
+ * P-partial reduce + residual-add + RMSNorm path.
+ *
+ * One rank, one GPU.  Every pointer is a DEVICE pointer to row-major,
+ * row-contiguous memory ([num_tokens, hidden_size], element stride 1, row
+ * stride hidden_size) unless stated otherwise.  Every call only ENQUEUES work
+ * on `stream` (a hipStream_t; NULL = the default stream) of the device that is
+ * current on the calling thread: no allocation, no host synchronisation, safe
+ * under stream capture.  Return value: TW_OK, or a negative TW_ERR_* code with
+ * a message retrievable from tw_last_error() on the same thread.  Nothing
+ * throws across this boundary.
+ *
+ * Arithmetic (identical for every entry point; the reference's CPU path,
+ * csrc/cpu/layernorm.cpp:44-88, with round-to-nearest-even stores):
+ *   S   = sum_{p=0}^{P-1} f32(partial_p)        fp32, fixed order p = 0..P-1
+ *   s   = S + f32(residual)                      fp32
+ *   r'  = bf16_rne(s)                            -> residual (in place)
+ *   inv = 1 / sqrt( sum_j s_j^2 / H + eps )      fp32, unrounded s
+ *   y   = bf16_rne( f32(r') * inv * f32(w) )     -> output
+ * Row results do not depend on num_tokens, on max_ctas or on which other rows
+ * are in the call.
+ */
+#ifndef TOKENWEAVE_AMD_H
+#define TOKENWEAVE_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TW_API __attribute__((visibility("default")))
+
+#define TW_OK 0
+#define TW_ERR_INVALID_ARGUMENT (-1) /* null pointer, negative size, bad P / rank */
+#define TW_ERR_ALIGNMENT (-2)        /* 16-byte alignment or H % 8 violated      */
+#define TW_ERR_DTYPE (-3)            /* dtype not supported by this entry point   */
+#define TW_ERR_LAUNCH (-4)           /* the HIP runtime refused the launch        */
+
+/* Element types of the baseline ops (the reference dispatches them with
+ * VLLM_DISPATCH_FLOATING_TYPES, csrc/dispatch_utils.h:14-21).  The *_cta and
+ * reduce entry points are bf16 only, like the reference's
+ * VLLM_BF16_DISPATCH_FLOATING_TYPES (csrc/dispatch_utils.h:23-27). */
+#define TW_DTYPE_BF16 0
+#define TW_DTYPE_F16 1
+#define TW_DTYPE_F32 2
+
+#define TW_MAX_PARTIALS 16
+
+/* Library version (major*10000 + minor*100 + patch). */
+TW_API int tw_version(void);
+
+/* Message for the last non-TW_OK return on this thread ("" if none). */
+TW_API const char* tw_last_error(void);
+
+/* Number of compute units of the current device (<0 on error). */
+TW_API int tw_num_compute_units(void);
+
+/* input <- RMSNorm(input + residual) * weight ; residual <- input + residual.
+ * Replaces ::fused_add_rms_norm (csrc/layernorm_kernels.cu:194-231, schema at
+ * csrc/torch_bindings.cpp:141-144; CPU twin csrc/cpu/layernorm.cpp:105-117).
+ * Any hidden_size and alignment are accepted: rows that are not 16-byte
+ * aligned or hidden_size % 8 != 0 take an element-wise kernel, as the
+ * reference's launcher does (layernorm_kernels.cu:223-230). */
+TW_API int tw_fused_add_rms_norm(void* input, void* residual, const void* weight,
+                          int64_t num_tokens, int64_t hidden_size,
+                          float epsilon, int dtype, void* stream);
+
+/* out <- RMSNorm(input) * weight.
+ * Replaces ::rms_norm (csrc/layernorm_kernels.cu:165-181, schema at
+ * csrc/torch_bindings.cpp:135-138; CPU twin csrc/cpu/layernorm.cpp:91-103). */
+TW_API int tw_rms_norm(void* out, const void* input, const void* weight,
+                int64_t num_tokens, int64_t hidden_size, float epsilon,
+                int dtype, void* stream);
+
+/* out <- input (the copy becomes the residual stream) ;
+ * input <- RMSNorm(input) * weight.
+ * Replaces ::rms_norm_inplace (csrc/tokenweave_fused_kernels.cu:186-202,
+ * schema at csrc/torch_bindings.cpp:147-150). */
+TW_API int tw_rms_norm_inplace(void* out, void* input, const void* weight,
+                        int64_t num_tokens, int64_t hidden_size, float epsilon,
+                        int dtype, void* stream);
+
+/* tw_fused_add_rms_norm on a grid capped at max_ctas workgroups that walk the
+ * rows with stride max_ctas (max_ctas <= 0: library default).  bf16 only;
+ * pointers must be 16-byte aligned and hidden_size % 8 == 0, else
+ * TW_ERR_ALIGNMENT.
+ * Replaces ::fused_add_rms_norm_cta (csrc/tokenweave_artifact_kernels.cu:
+ * 717-754, schema at csrc/torch_bindings.cpp:160-164). */
+TW_API int tw_fused_add_rms_norm_cta(void* input, void* residual, const void* weight,
+                              int64_t num_tokens, int64_t hidden_size,
+                              int max_ctas, float epsilon, void* stream);
+
+/* The fused op restricted to one GPU, general form.
+ *   partials : HOST array of P device pointers, each [num_tokens, hidden_size]
+ *              bf16 (this rank's row shard of every tensor-parallel partial sum)
+ *   y        : [num_tokens, hidden_size] bf16 output; may alias any partials[p]
+ *   residual : read and overwritten with r'
+ * 1 <= P <= TW_MAX_PARTIALS.  bf16; 16-byte alignment and H % 8 == 0 required.
+ * This is the body of fused_rs_ln_ag_cta_kernel
+ * (csrc/tokenweave_fused_kernels.cu:106-152) with the switch-side
+ * multimem.ld_reduce replaced by P loads from local HBM. */
+TW_API int tw_reduce_add_rms_norm(const void* const* partials, int num_partials,
+                           void* y, void* residual, const void* weight,
+                           int64_t num_tokens, int64_t hidden_size,
+                           int max_ctas, float epsilon, void* stream);
+
+/* Same op with the reference's argument list.  `mcptr` is the device address
+ * of this rank's row shard inside partial buffer 0; partial p lives at
+ * mcptr + p * peer_stride_bytes (the one-GPU stand-in for "the same offset in
+ * every peer's symmetric buffer").  y is written to `input`, which normally is
+ * the shard of partial `rank` (mcptr + rank * peer_stride_bytes), as the
+ * reference stores y over its own staging rows.  signal pads do not exist on
+ * one GPU and are not part of this ABI.
+ * Replaces ::fused_rs_ln_cta (csrc/tokenweave_artifact_kernels.cu:772-813,
+ * schema at csrc/torch_bindings.cpp:166-171). */
+TW_API int tw_fused_rs_ln_cta(void* input, void* residual, const void* weight,
+                       uint64_t mcptr, int64_t peer_stride_bytes, int rank,
+                       int world_size, int max_ctas, float epsilon,
+                       int64_t num_tokens, int64_t hidden_size, void* stream);
+
+/* Identical to tw_fused_rs_ln_cta on one GPU: the all-gather that distinguishes
+ * the reference op is the store of y to the peers, and there are none.
+ * Replaces ::fused_rs_ln_ag_cta (csrc/tokenweave_fused_kernels.cu:220-261,
+ * schema at csrc/torch_bindings.cpp:152-157). */
+TW_API int tw_fused_rs_ln_ag_cta(void* input, void* residual, const void* weight,
+                          uint64_t mcptr, int64_t peer_stride_bytes, int rank,
+                          int world_size, int max_ctas, float epsilon,
+                          int64_t num_tokens, int64_t hidden_size,
+                          void* stream);
+
+/* out[M, N] = a[M, K] * b[N, K]^T, bf16 in, fp32 accumulate on MFMA, bf16 out.
+ * `ldc` is the row stride of out in elements (>= N), so the result can land in
+ * a row slice of a wider staging buffer.  Required: K % 8 == 0, N % 4 == 0,
+ * ldc % 4 == 0, 16-byte aligned a and b, 8-byte aligned out.  max_cus > 0
+ * limits the grid to that many workgroups so a concurrent kernel keeps the
+ * remaining compute units.
+ * Replaces UnquantizedLinearMethod.apply_inplace = torch.matmul(x, W.t(), out=)
+ * (vllm/model_executor/layers/linear.py:203-228) for the row-parallel o_proj /
+ * down_proj that produces one rank's partial sum. */
+TW_API int tw_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M,
+                    int64_t N, int64_t K, int64_t ldc, int max_cus,
+                    void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TOKENWEAVE_AMD_H */

@@ -1,0 +1,152 @@
+/*
+ * TEST INFRASTRUCTURE ONLY.  CPU restatement of the reference's fp32-accumulate
+ * residual-add + RMSNorm path, extended to P partial-sum buffers.  Only tests,
+ * the smoke check and the benchmark's cpu_baseline leg may load this library;
+ * the product (tokenweave_amd) never does.
+ *
+ * Reference followed, line by line:
+ *   csrc/cpu/layernorm.cpp:44-88   fused_add_rms_norm_impl  (operation order,
+ *                                  which value is squared, which is re-read)
+ *   csrc/cpu/layernorm.cpp:4-41    rms_norm_impl
+ *   csrc/cpu/cpu_types_x86.hpp:208-241  FP32Vec8: 8 independent fp32 lane
+ *                                  accumulators, reduce_sum = lanes 0..7 in order
+ *   csrc/cpu/cpu_types_x86.hpp:229-231  bf16 -> f32 is a 16-bit left shift
+ *   csrc/cpu/cpu_types_x86.hpp:647-698  f32 -> bf16: round-to-nearest-even when
+ *                                  built with AVX512-BF16, truncation otherwise
+ *   csrc/custom_all_reduce.cuh:286-294  P-way sum: fp32, fixed order p = 0..P-1,
+ *                                  one down-cast at the end
+ *   csrc/tokenweave_fused_kernels.cu:37-72  rms_norm_inplace (copy + normalise)
+ *
+ * Pinned by (tests/test_oracle_*.py): bit equality with the reference's own
+ * layernorm.cpp compiled from its sources (oracle/_ref, truncating build) on the
+ * reference's test grid; closed forms (constant / one-hot / zero rows); an
+ * independent numpy fp32 restatement of RMSNorm.forward_native; float64 witness.
+ *
+ * Every function is built with -ffp-contract=off: the reference's vector code is
+ * separate multiplies and adds (no FMA in its AVX2 build).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+
+#define TW_ROUND_RNE 0   /* AVX512-BF16 build of the reference */
+#define TW_ROUND_TRUNC 1 /* every other x86 build of the reference */
+
+static inline float bf16_to_f32(uint16_t v) {
+  uint32_t u = (uint32_t)v << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+static inline uint16_t f32_to_bf16(float f, int mode) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  if (mode == TW_ROUND_TRUNC) return (uint16_t)(u >> 16);
+  if ((u & 0x7fffffffu) > 0x7f800000u) /* NaN: keep it quiet, as vcvtneps2bf16 */
+    return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+/* Row kernel shared by every entry point.
+ *   np == 0 : s = x            (rms_norm: nothing added, nothing written back)
+ *   np >= 1 : s = (((p0 + p1) + ...) + p_{np-1}) + r   in fp32, r optional
+ * sum of squares uses the UNROUNDED fp32 s (layernorm.cpp:65-67);
+ * the normalised output re-reads the ROUNDED residual (layernorm.cpp:78-83). */
+static void row_reduce_add_norm(const uint16_t* const* parts, int np,
+                                int64_t row_off, uint16_t* res_row,
+                                uint16_t* y_row, const uint16_t* w, float eps,
+                                int H, int mode) {
+  float lane[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int j = 0; j < H; j += 8) {
+    for (int k = 0; k < 8; ++k) {
+      float s = bf16_to_f32(parts[0][row_off + j + k]);
+      for (int p = 1; p < np; ++p) s = s + bf16_to_f32(parts[p][row_off + j + k]);
+      if (res_row) s = s + bf16_to_f32(res_row[j + k]);
+      float sq = s * s;
+      lane[k] = lane[k] + sq;
+      if (res_row) res_row[j + k] = f32_to_bf16(s, mode);
+    }
+  }
+  float ss = 0.0f;
+  for (int k = 0; k < 8; ++k) ss += lane[k];
+  float mean = ss / (float)H;
+  float inv = 1.0f / sqrtf(mean + eps);
+  const uint16_t* src = res_row ? res_row : parts[0] + row_off;
+  /* y_row may alias parts[*] + row_off: all reads of the row are done. */
+  for (int j = 0; j < H; ++j) {
+    float t = bf16_to_f32(src[j]) * inv;
+    t = t * bf16_to_f32(w[j]);
+    y_row[j] = f32_to_bf16(t, mode);
+  }
+}
+
+/* x <- norm(x + r) * w ; r <- x + r.  layernorm.cpp:44-88. */
+int tw_oracle_fused_add_rms_norm(uint16_t* x, uint16_t* r, const uint16_t* w,
+                                 int64_t T, int64_t H, float eps, int mode) {
+  if (H % 8 != 0 || H <= 0 || T < 0) return -1; /* TORCH_CHECK layernorm.cpp:52 */
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < T; ++i) {
+    const uint16_t* parts[1] = {x};
+    row_reduce_add_norm(parts, 1, i * H, r + i * H, x + i * H, w, eps, (int)H, mode);
+  }
+  return 0;
+}
+
+/* y <- norm(sum_p partial_p + r) * w ; r <- sum_p partial_p + r.
+ * y may alias any partials[p].  P=1 with y == partials[0] is the function above. */
+int tw_oracle_reduce_add_rms_norm(const uint16_t* const* partials, int P,
+                                  uint16_t* y, uint16_t* r, const uint16_t* w,
+                                  int64_t T, int64_t H, float eps, int mode) {
+  if (H % 8 != 0 || H <= 0 || T < 0 || P < 1 || P > 64) return -1;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < T; ++i)
+    row_reduce_add_norm(partials, P, i * H, r + i * H, y + i * H, w, eps, (int)H, mode);
+  return 0;
+}
+
+/* out <- norm(x) * w.  layernorm.cpp:4-41. */
+int tw_oracle_rms_norm(uint16_t* out, const uint16_t* x, const uint16_t* w,
+                       int64_t T, int64_t H, float eps, int mode) {
+  if (H % 8 != 0 || H <= 0 || T < 0) return -1; /* TORCH_CHECK layernorm.cpp:11 */
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < T; ++i) {
+    const uint16_t* parts[1] = {x};
+    row_reduce_add_norm(parts, 0, i * H, 0, out + i * H, w, eps, (int)H, mode);
+  }
+  return 0;
+}
+
+/* out <- x (becomes the residual) ; x <- norm(x) * w.
+ * tokenweave_fused_kernels.cu:37-72 with the CPU path's single rounding. */
+int tw_oracle_rms_norm_inplace(uint16_t* out, uint16_t* x, const uint16_t* w,
+                               int64_t T, int64_t H, float eps, int mode) {
+  if (H % 8 != 0 || H <= 0 || T < 0) return -1;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < T; ++i) {
+    memcpy(out + i * H, x + i * H, (size_t)H * 2);
+    const uint16_t* parts[1] = {x};
+    row_reduce_add_norm(parts, 0, i * H, 0, x + i * H, w, eps, (int)H, mode);
+  }
+  return 0;
+}
+
+/* out[M,N] = bf16( sum_k f32(a[M,K]) * f32(b[N,K]) ), fp32 accumulate, k ascending.
+ * Semantics of torch.matmul(x, W.t(), out=) at
+ * vllm/model_executor/layers/linear.py:224 (accumulation order is the BLAS's
+ * there; this is the plain order, compared under tolerance only). */
+int tw_oracle_gemm_bf16_nt(uint16_t* out, const uint16_t* a, const uint16_t* b,
+                           int64_t M, int64_t N, int64_t K, int mode) {
+  if (M < 0 || N <= 0 || K <= 0) return -1;
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) {
+      float acc = 0.0f;
+      for (int64_t k = 0; k < K; ++k)
+        acc = acc + bf16_to_f32(a[m * K + k]) * bf16_to_f32(b[n * K + k]);
+      out[m * N + n] = f32_to_bf16(acc, mode);
+    }
+  }
+  return 0;
+}

@@ -1,0 +1,113 @@
+"""The weave configuration on a real GPU: the bf16 MFMA GEMM that produces a
+rank's partial sum, and the two-stream step that overlaps it with the fused norm.
+
+GEMM parity is against fp32 arithmetic on the CPU at rtol 1.6e-2 / atol 1e-2 (no
+reference test pins torch.matmul's accumulation order for this call)."""
+import numpy as np
+import pytest
+import torch
+
+import tokenweave_amd as tw
+from helpers import ATOL, RTOL, to_bits
+from tokenweave_amd import _custom_ops as ops
+from tokenweave_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def cpu_gemm(a, b):
+    return (a.float().cpu() @ b.float().cpu().t())
+
+
+def check(out, a, b, what):
+    want = cpu_gemm(a, b)
+    torch.testing.assert_close(out.float().cpu(), want, rtol=RTOL, atol=ATOL, msg=lambda m: f"{what}: {m}")
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 128, 64), (100, 128, 64), (129, 256, 128), (128, 136, 72),
+                                   (257, 384, 1024), (333, 8192, 1024)])
+def test_gemm_shapes_and_tails(M, N, K):
+    print(f"[case] gemm M={M} N={N} K={K}", flush=True)
+    g = wl.make_gemm_inputs(M, N, K, DEV, seed=M * 7 + N)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16_nt(out, g.a, g.b)
+    torch.cuda.synchronize()
+    check(out, g.a, g.b, f"{M}x{N}x{K}")
+
+
+def test_gemm_small_against_c_oracle(oracle):
+    g = wl.make_gemm_inputs(70, 96, 160, DEV, seed=5, weight_std=1.0)
+    out = torch.empty((70, 96), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16_nt(out, g.a, g.b)
+    torch.cuda.synchronize()
+    want = oracle.gemm_bf16_nt(to_bits(g.a), to_bits(g.b))
+    got = to_bits(out)
+    f = lambda u: (u.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    assert np.all(np.abs(f(got) - f(want)) <= ATOL + RTOL * np.abs(f(want)))
+
+
+def test_gemm_weave_shape_into_a_staging_slice_with_cu_cap():
+    """Config 5's GEMM: [2458, 1024] x [8192, 1024]^T written into rows of a wider
+    staging buffer, once uncapped and once on a capped grid; both must agree bitwise."""
+    g = wl.make_gemm_inputs(device=DEV)
+    M, N = g.a.shape[0], g.b.shape[0]
+    stage = torch.zeros((wl.C5_TOTAL_TOKENS, N), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16_nt(stage[:M], g.a, g.b)
+    capped = torch.zeros_like(stage)
+    ops.gemm_bf16_nt(capped[:M], g.a, g.b, max_cus=96)
+    torch.cuda.synchronize()
+    check(stage[:M], g.a, g.b, "weave gemm")
+    assert torch.equal(stage, capped)
+    assert not stage[M:].any(), "rows of the other split were touched"
+
+
+def test_gemm_output_with_wide_row_stride():
+    g = wl.make_gemm_inputs(65, 128, 64, DEV, seed=9)
+    wide = torch.zeros((65, 256), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16_nt(wide[:, :128], g.a, g.b)
+    torch.cuda.synchronize()
+    check(wide[:, :128], g.a, g.b, "ldc")
+    assert not wide[:, 128:].any()
+
+
+def test_weave_step_equals_serial_execution():
+    """GEMM of split A on the current stream while split B's fused norm runs on a
+    second stream (tokenweave_utils.py:236-260): same bits as running them in turn."""
+    ws, H, T = 8, 8192, 512
+    Ta = tw.tokenweave_split_size(T)  # 256
+    Tb = T - Ta
+    cfg = wl.C5_NORM.with_tokens(Tb)
+    inp = wl.make_norm_inputs(cfg, DEV)
+    g = wl.make_gemm_inputs(Ta, H, 1024, DEV)
+    layer = tw.RMSNorm(H, eps=cfg.eps, dtype=torch.bfloat16).to(DEV)
+    layer.weight.data.copy_(inp.weight)
+
+    def setup():
+        buf = tw.PartialsBuffer(ws, T, H, rank=2, device=DEV)
+        buf.storage.zero_()
+        buf.storage[:, Ta:] = inp.staging
+        residual = torch.zeros(T, H, dtype=torch.bfloat16, device=DEV)
+        residual[Ta:] = inp.residual
+        return buf, residual
+
+    def norm(buf, residual):
+        layer(buf.local[Ta:], residual[Ta:], MAX_CTAS=64, fused_ar=True, symm_mem_hdl=buf, rank=2,
+              world_size=ws, offset=buf.offset_of_row(Ta))
+
+    def gemm(buf):
+        ops.gemm_bf16_nt(buf.local[:Ta], g.a, g.b, max_cus=192)
+
+    buf1, res1 = setup()
+    gemm(buf1)
+    norm(buf1, res1)
+    torch.cuda.synchronize()
+    buf2, res2 = setup()
+    side = torch.cuda.Stream()
+    for _ in range(3):  # the step is idempotent on split A and we reset split B each time
+        buf2.storage[:, Ta:] = inp.staging
+        res2[Ta:] = inp.residual
+        tw.weave_norm_gemm(lambda: gemm(buf2), lambda: norm(buf2, res2), side)
+        torch.cuda.synchronize()
+        assert torch.equal(buf1.storage, buf2.storage) and torch.equal(res1, res2)
+    check(buf2.local[:Ta], g.a, g.b, "weave gemm split")

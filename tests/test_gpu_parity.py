@@ -1,0 +1,328 @@
+"""Parity of the HIP path (through the C ABI) with the CPU checker, on a real GPU.
+
+Bar: rtol 1.6e-2 / atol 1e-2 on y and on the updated residual (helpers.RTOL/ATOL);
+on top of it the residual must be bit-exact and y within one bf16 ulp.
+"""
+import numpy as np
+import pytest
+import torch
+
+import tokenweave_amd as tw
+from helpers import assert_close_bits, assert_parity, from_bits, to_bits, ulp_distance
+from tokenweave_amd import _custom_ops as ops
+from tokenweave_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def run_oracle(oracle, inp):
+    parts = [to_bits(p) for p in inp.partials]
+    r = to_bits(inp.residual)
+    y, r = oracle.reduce_add_rms_norm(parts, r, to_bits(inp.weight), inp.cfg.eps)
+    return y, r
+
+
+def run_hip(inp, max_ctas=None, alias_rank=None):
+    parts = [p.clone() for p in inp.partials]
+    res = inp.residual.clone()
+    out = parts[alias_rank] if alias_rank is not None else torch.empty_like(res)
+    ops.reduce_add_rms_norm(parts, out, res, inp.weight, inp.cfg.eps, max_ctas)
+    torch.cuda.synchronize()
+    return to_bits(out), to_bits(res), parts
+
+
+# ---------------------------------------------------------------------------
+# the benchmark configurations, full size
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("name", list(wl.norm_configs()))
+def test_benchmark_config_parity(oracle, name):
+    cfg = wl.norm_configs()[name]
+    print(f"[case] {name} P={cfg.P} T={cfg.T} H={cfg.H}", flush=True)
+    inp = wl.make_norm_inputs(cfg, DEV)
+    y_want, r_want = run_oracle(oracle, inp)
+    if cfg.P == 1:  # config 1 is the reference's fused_add_rms_norm call itself
+        x, res = inp.partials[0].clone(), inp.residual.clone()
+        ops.fused_add_rms_norm(x, res, inp.weight, cfg.eps)
+        torch.cuda.synchronize()
+        y_got, r_got = to_bits(x), to_bits(res)
+    else:
+        y_got, r_got, _ = run_hip(inp, alias_rank=0)
+    assert_parity(y_got, r_got, y_want, r_want, name)
+
+
+def test_golden_vectors_from_the_reference_cpu_build(oracle):
+    """Inputs/outputs produced by the reference's compiled layernorm.cpp (truncating
+    store): the HIP path (RNE store) must sit inside the tolerance of the path, and
+    agree with the RNE checker tightly, on the same inputs."""
+    import os
+    npz = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_fused_add_rms_norm.npz"))
+    names = sorted({k.split(".")[0] for k in npz.files})
+    for n in names:
+        print(f"[case] golden {n}", flush=True)
+        x, r, w = npz[n + ".x"], npz[n + ".r"], npz[n + ".w"]
+        eps = float(npz[n + ".eps"])
+        xd, rd, wd = from_bits(x, DEV), from_bits(r, DEV), from_bits(w, DEV)
+        ops.fused_add_rms_norm(xd, rd, wd, eps)
+        torch.cuda.synchronize()
+        y_got, r_got = to_bits(xd), to_bits(rd)
+        assert_close_bits(r_got, npz[n + ".r_ref"], n + " residual vs reference build")
+        assert_close_bits(y_got, npz[n + ".y_ref"], n + " y vs reference build")
+        xo, ro = x.copy(), r.copy()
+        oracle.fused_add_rms_norm(xo, ro, w, eps)
+        assert np.array_equal(r_got, ro), n
+        assert ulp_distance(y_got, xo).max() <= 1, n
+    npz = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_rms_norm.npz"))
+    for n in sorted({k.split(".")[0] for k in npz.files}):
+        x, w, eps = npz[n + ".x"], npz[n + ".w"], float(npz[n + ".eps"])
+        xd, wd = from_bits(x, DEV), from_bits(w, DEV)
+        out = torch.empty_like(xd)
+        ops.rms_norm(out, xd, wd, eps)
+        torch.cuda.synchronize()
+        assert_close_bits(to_bits(out), npz[n + ".y_ref"], n + " rms_norm vs reference build")
+        assert ulp_distance(to_bits(out), oracle.rms_norm(x, w, eps)).max() <= 1, n
+        assert np.array_equal(to_bits(xd), x), "rms_norm must not modify its input"
+
+
+# ---------------------------------------------------------------------------
+# the reference's own unit-test grid (tests/kernels/test_layernorm.py:11-57)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.half, torch.bfloat16, torch.float])
+@pytest.mark.parametrize("add_residual", [False, True])
+@pytest.mark.parametrize("hidden_size", [8, 768, 769, 770, 771, 5120, 5124, 5125, 5126, 8192, 8199])
+@pytest.mark.parametrize("num_tokens", [7, 83, 4096])
+def test_reference_unit_test_grid(num_tokens, hidden_size, add_residual, dtype):
+    torch.manual_seed(0)
+    layer = tw.RMSNorm(hidden_size).to(dtype=dtype, device=DEV)
+    layer.weight.data.normal_(mean=1.0, std=0.1)
+    scale = 1 / (2 * hidden_size)
+    x = torch.randn(num_tokens, hidden_size, dtype=dtype, device=DEV) * scale
+    residual = torch.randn_like(x) * scale if add_residual else None
+    ref_out = layer.forward_native(x, residual)
+    out = layer(x, residual)
+    if add_residual:
+        assert out[0] is x and out[1] is residual  # mutated in place, same objects returned
+        torch.testing.assert_close(out[0], ref_out[0], atol=1e-2, rtol=1e-2)
+        torch.testing.assert_close(out[1], ref_out[1], atol=1e-2, rtol=1e-2)
+    else:
+        torch.testing.assert_close(out, ref_out, atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("T,H", [(7, 8), (83, 768), (83, 5120), (4096, 8192), (5, 16384), (3, 32768), (2, 40960)])
+def test_bf16_grid_against_checker_tight(oracle, T, H):
+    torch.manual_seed(1)
+    x = torch.randn(T, H, device=DEV).to(torch.bfloat16)
+    r = torch.randn(T, H, device=DEV).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(H, device=DEV)).to(torch.bfloat16)
+    xo, ro = to_bits(x), to_bits(r)
+    oracle.fused_add_rms_norm(xo, ro, to_bits(w), 1e-5)
+    x2 = x.clone()
+    ops.fused_add_rms_norm(x, r, w, 1e-5)
+    torch.cuda.synchronize()
+    assert_parity(to_bits(x), to_bits(r), xo, ro, f"T{T} H{H}")
+    # rms_norm and rms_norm_inplace on the same rows
+    want = oracle.rms_norm(to_bits(x2), to_bits(w), 1e-5)
+    out = torch.empty_like(x2)
+    ops.rms_norm(out, x2, w, 1e-5)
+    keep = x2.clone()
+    copy = torch.zeros_like(x2)
+    ops.rms_norm_inplace(copy, x2, w, 1e-5)
+    torch.cuda.synchronize()
+    assert ulp_distance(to_bits(out), want).max() <= 1
+    assert torch.equal(copy, keep) and torch.equal(x2, out)
+
+
+@pytest.mark.parametrize("P", [1, 2, 3, 4, 5, 7, 8, 16])
+@pytest.mark.parametrize("H", [64, 6144, 8192, 16384])
+def test_partial_counts_and_widths(oracle, P, H):
+    cfg = wl.NormConfig("sweep", P=P, T=37, H=H, eps=1e-5, seed=4242 + P, partial_std=P ** -0.5)
+    inp = wl.make_norm_inputs(cfg, DEV)
+    y_want, r_want = run_oracle(oracle, inp)
+    y_got, r_got, _ = run_hip(inp)
+    assert_parity(y_got, r_got, y_want, r_want, f"P{P} H{H}")
+
+
+# ---------------------------------------------------------------------------
+# launch-shape independence, aliasing, in-place contract
+# ---------------------------------------------------------------------------
+def test_rows_do_not_depend_on_grid_cap_or_batch(oracle):
+    cfg = wl.C2.with_tokens(300)
+    inp = wl.make_norm_inputs(cfg, DEV)
+    y0, r0, _ = run_hip(inp)
+    for cap in (1, 2, 7, 64, 299, 300, 5000):
+        y, r, _ = run_hip(inp, max_ctas=cap)
+        assert np.array_equal(y, y0) and np.array_equal(r, r0), f"max_ctas={cap}"
+    sub = wl.NormInputs(cfg, [p[100:117].contiguous() for p in inp.partials],
+                        inp.residual[100:117].contiguous(), inp.weight)
+    y, r, _ = run_hip(sub)
+    assert np.array_equal(y, y0[100:117]) and np.array_equal(r, r0[100:117])
+    perm = torch.randperm(cfg.T, device=DEV)
+    shuf = wl.NormInputs(cfg, [p[perm].contiguous() for p in inp.partials],
+                         inp.residual[perm].contiguous(), inp.weight)
+    y, r, _ = run_hip(shuf)
+    assert np.array_equal(y, y0[perm.cpu().numpy()])
+
+
+@pytest.mark.parametrize("rank", [0, 3, 7])
+def test_output_may_alias_any_partial(rank):
+    inp = wl.make_norm_inputs(wl.C2.with_tokens(64), DEV)
+    y0, r0, _ = run_hip(inp)
+    y, r, parts = run_hip(inp, alias_rank=rank)
+    assert np.array_equal(y, y0) and np.array_equal(r, r0)
+    for p in range(8):
+        if p != rank:
+            assert torch.equal(parts[p], inp.partials[p]), f"partial {p} was modified"
+
+
+def test_zero_partials_reduce_to_fused_add_rms_norm():
+    inp = wl.make_norm_inputs(wl.C1.with_tokens(33), DEV)
+    x, r = inp.partials[0].clone(), inp.residual.clone()
+    ops.fused_add_rms_norm(x, r, inp.weight, 1e-5)
+    zeros = [torch.zeros_like(x) for _ in range(7)]
+    out, r8 = torch.empty_like(x), inp.residual.clone()
+    ops.reduce_add_rms_norm([inp.partials[0]] + zeros, out, r8, inp.weight, 1e-5)
+    x2, r2 = inp.partials[0].clone(), inp.residual.clone()
+    ops.fused_add_rms_norm_cta(x2, r2, inp.weight, 5, 1e-5)
+    torch.cuda.synchronize()
+    assert torch.equal(out, x) and torch.equal(r8, r)
+    assert torch.equal(x2, x) and torch.equal(r2, r)
+
+
+def test_closed_forms_on_device():
+    H, eps = 8192, 1e-5
+    w = torch.full((H,), 1.25, dtype=torch.bfloat16, device=DEV)
+    x = torch.zeros(3, H, dtype=torch.bfloat16, device=DEV)
+    r = torch.zeros_like(x)
+    x[1] = 0.5
+    x[2, 4097] = 8.0
+    ops.fused_add_rms_norm(x, r, w, eps)
+    torch.cuda.synchronize()
+    xf = x.float().cpu()
+    assert (xf[0] == 0).all() and torch.isfinite(xf).all()
+    want = torch.tensor(0.5 * (1.0 / np.sqrt(np.float32(0.25) + np.float32(eps))) * 1.25).to(torch.bfloat16).float()
+    assert (xf[1] == want).all()
+    inv = 1.0 / np.sqrt(64.0 / H + eps)
+    assert abs(xf[2, 4097] - 8.0 * inv * 1.25) <= 2 ** -7 * 8.0 * inv * 1.25
+    assert xf[2].count_nonzero() == 1
+    assert (r[1].float() == 0.5).all().item()
+
+
+# ---------------------------------------------------------------------------
+# the reference's call site: RMSNorm(fused_ar=True) via fused_allreduce_layernorm
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("fused_kw", ["fused_ar", "fused_rs"])
+def test_call_site_through_partials_buffer(oracle, fused_kw):
+    ws, T, H, eps = 8, 64, 8192, 1e-5
+    torch.manual_seed(7)
+    layer = tw.RMSNorm(H, eps=eps, dtype=torch.bfloat16).to(DEV)
+    layer.weight.data.normal_(mean=1.0, std=0.1)
+    residual0 = torch.randn(T, H, device=DEV).to(torch.bfloat16)
+    stage0 = (torch.randn(ws, T + 5, H, device=DEV) * ws ** -0.5).to(torch.bfloat16)
+    for rank in (0, 5):
+        buf = tw.PartialsBuffer(ws, T + 5, H, rank=rank, device=DEV)
+        buf.storage.copy_(stage0)
+        residual = residual0.clone()
+        hidden_states = buf.hidden_states(T)
+        if fused_kw == "fused_ar":
+            tw.fused_allreduce_layernorm(layer, hidden_states, residual, buf, T // ws, rank, ws, 16)
+        else:
+            s, e = tw.shard_bounds(T, rank, ws)
+            layer(hidden_states[s:e], residual[s:e], MAX_CTAS=4, fused_rs=True, symm_mem_hdl=buf,
+                  rank=rank, world_size=ws, offset=buf.offset_of_row(s))
+        torch.cuda.synchronize()
+        s, e = tw.shard_bounds(T, rank, ws)
+        parts = [to_bits(stage0[p, s:e]) for p in range(ws)]
+        y_want, r_want = oracle.reduce_add_rms_norm(parts, to_bits(residual0[s:e]), to_bits(layer.weight.data), eps)
+        assert_parity(to_bits(hidden_states[s:e]), to_bits(residual[s:e]), y_want, r_want, f"rank {rank}")
+        # nothing outside this rank's rows of its own slot changed
+        after = buf.storage.clone()
+        after[rank, s:e] = stage0[rank, s:e]
+        assert torch.equal(after, stage0)
+        keep = residual.clone()
+        keep[s:e] = residual0[s:e]
+        assert torch.equal(keep, residual0)
+
+
+def test_ragged_shards_cover_the_batch_exactly_once(oracle):
+    ws, H = 8, 8192
+    cfg = wl.C3.with_tokens(333)
+    inp = wl.make_norm_inputs(cfg, DEV)
+    y_want, r_want = run_oracle(oracle, inp)
+    layer = tw.RMSNorm(H, eps=cfg.eps, dtype=torch.bfloat16).to(DEV)
+    layer.weight.data.copy_(inp.weight)
+    for mode in ("floor", "ceil"):
+        residual = inp.residual.clone()
+        y_all = torch.empty_like(residual)
+        for rank in range(ws):   # each simulated rank normalises its own rows
+            buf = tw.PartialsBuffer(ws, cfg.T, H, rank=rank, device=DEV)
+            buf.storage.copy_(inp.staging)
+            rng = tw.shard_bounds(cfg.T, rank, ws, mode)
+            tw.fused_allreduce_layernorm(layer, buf.hidden_states(cfg.T), residual, buf, 0, rank, ws, 64,
+                                         row_range=rng)
+            y_all[rng[0]:rng[1]] = buf.hidden_states(cfg.T)[rng[0]:rng[1]]
+        torch.cuda.synchronize()
+        assert_parity(to_bits(y_all), to_bits(residual), y_want, r_want, mode)
+
+
+# ---------------------------------------------------------------------------
+# streams and argument errors with device tensors
+# ---------------------------------------------------------------------------
+def test_runs_on_the_current_torch_stream(oracle):
+    inp = wl.make_norm_inputs(wl.C2.with_tokens(128), DEV)
+    y0, r0, _ = run_hip(inp)
+    side = torch.cuda.Stream()
+    parts = [p.clone() for p in inp.partials]
+    res, out = inp.residual.clone(), torch.empty_like(inp.residual)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        ops.reduce_add_rms_norm(parts, out, res, inp.weight, inp.cfg.eps)
+    side.synchronize()
+    assert np.array_equal(to_bits(out), y0) and np.array_equal(to_bits(res), r0)
+
+
+def test_argument_errors_on_device_tensors():
+    H = 64
+    x = torch.zeros(8, H, dtype=torch.bfloat16, device=DEV)
+    w = torch.ones(H, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="row-contiguous"):
+        ops.fused_add_rms_norm(x[:, ::2], x[:, ::2].clone(), w[:32], 1e-5)
+    with pytest.raises(RuntimeError, match="same shape"):
+        ops.fused_add_rms_norm(x, x[:4].clone(), w, 1e-5)
+    with pytest.raises(RuntimeError, match="expected hidden_size"):
+        ops.fused_add_rms_norm(x, x.clone(), w[:32].clone(), 1e-5)
+    flat = torch.zeros(8 * H + 8, dtype=torch.bfloat16, device=DEV)
+    mis = flat[1:1 + 8 * H].view(8, H)      # 2-byte offset: not 16-byte aligned
+    with pytest.raises(RuntimeError, match="16-byte aligned"):
+        ops.fused_add_rms_norm_cta(mis, x.clone(), w, 4, 1e-5)
+    with pytest.raises(RuntimeError, match="16-byte aligned"):
+        ops.reduce_add_rms_norm([x, mis], x.clone(), x.clone(), w, 1e-5)
+    buf = tw.PartialsBuffer(4, 8, H, device=DEV)
+    with pytest.raises(RuntimeError, match="Invalid rank"):
+        ops.fused_rs_ln_ag_cta(buf.local, x.clone(), w, buf.multicast_ptr, 0, 4, 4, 8, 1e-5)
+    with pytest.raises(RuntimeError, match="not inside slot 0"):
+        ops.fused_rs_ln_ag_cta(buf.local, x.clone(), w, x.data_ptr(), 0, 0, 4, 8, 1e-5)
+    torch.cuda.synchronize()
+
+
+def test_misaligned_rows_take_the_elementwise_kernel(oracle):
+    """The baseline op accepts what the vector kernel cannot
+    (csrc/layernorm_kernels.cu:223-230)."""
+    T, H = 9, 72
+    torch.manual_seed(3)
+    flat = torch.randn(T * H + 8, device=DEV).to(torch.bfloat16)
+    x = flat[1:1 + T * H].view(T, H)
+    r = torch.randn(T, H, device=DEV).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(H, device=DEV)).to(torch.bfloat16)
+    xo, ro = to_bits(x), to_bits(r)
+    oracle.fused_add_rms_norm(xo, ro, to_bits(w), 1e-5)
+    ops.fused_add_rms_norm(x, r, w, 1e-5)
+    torch.cuda.synchronize()
+    assert_parity(to_bits(x), to_bits(r), xo, ro, "misaligned", max_y_mismatch=2e-2)
+
+
+def test_empty_batch_is_a_no_op():
+    x = torch.zeros(0, 8192, dtype=torch.bfloat16, device=DEV)
+    w = torch.ones(8192, dtype=torch.bfloat16, device=DEV)
+    ops.fused_add_rms_norm(x, x.clone(), w, 1e-5)
+    ops.reduce_add_rms_norm([x, x.clone()], x.clone(), x.clone(), w, 1e-5)
+    torch.cuda.synchronize()

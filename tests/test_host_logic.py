@@ -1,0 +1,158 @@
+"""Host-side mirror of the reference's Python interface for the path: schema
+strings, argument validation, row sharding, split arithmetic.  CPU only."""
+import pytest
+import torch
+
+import tokenweave_amd as tw
+from tokenweave_amd import _custom_ops as ops
+from tokenweave_amd import workloads as wl
+
+
+def test_schema_strings_are_the_reference_ones():
+    # csrc/torch_bindings.cpp:135-171
+    assert ops.SCHEMAS["fused_add_rms_norm"] == (
+        "fused_add_rms_norm(Tensor! input, Tensor! residual, Tensor weight, float epsilon) -> ()")
+    assert ops.SCHEMAS["rms_norm"] == "rms_norm(Tensor! result, Tensor input, Tensor weight, float epsilon) -> ()"
+    assert ops.SCHEMAS["fused_rs_ln_ag_cta"] == (
+        "fused_rs_ln_ag_cta(Tensor! input, Tensor! residual, Tensor weight, int mcptr, int signal_pads, "
+        "int rank, int world_size, int MAX_CTAS, float epsilon) -> ()")
+    for name in ops.SCHEMAS:
+        op = getattr(torch.ops.tokenweave_amd, name)
+        schema = op.default._schema
+        assert schema.name == f"tokenweave_amd::{name}"
+        assert len(schema.returns) == 0
+        assert schema.arguments[0].alias_info is not None and schema.arguments[0].alias_info.is_write
+
+
+def test_ops_refuse_cpu_tensors_loudly():
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    w = torch.ones(64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        ops.fused_add_rms_norm(x, x.clone(), w, 1e-5)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        torch.ops.tokenweave_amd.rms_norm(x.clone(), x, w, 1e-5)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.reduce_add_rms_norm([x], x.clone(), x.clone(), w, 1e-5)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        tw.RMSNorm(64, dtype=torch.bfloat16)(x, x.clone())
+
+
+def test_dtype_errors_use_dispatch_wording():
+    x = torch.zeros(4, 64, dtype=torch.float64)
+    with pytest.raises(NotImplementedError, match="not implemented for"):
+        ops.fused_add_rms_norm(x, x.clone(), torch.ones(64, dtype=torch.float64), 1e-5)
+    h = torch.zeros(4, 64, dtype=torch.float16)
+    with pytest.raises(NotImplementedError, match="fused_add_rms_norm_cta_kernel"):
+        ops.fused_add_rms_norm_cta(h, h.clone(), torch.ones(64, dtype=torch.float16), 8, 1e-5)
+
+
+def test_shard_bounds():
+    assert tw.shard_bounds(2048, 3, 8) == (768, 1024)
+    with pytest.raises(AssertionError, match="Mismatch in token count"):
+        tw.shard_bounds(3001, 0, 8)
+    with pytest.raises(AssertionError, match="Invalid rank"):
+        tw.shard_bounds(2048, 8, 8)
+    floor = [tw.shard_bounds(3001, r, 8, "floor") for r in range(8)]
+    ceil = [tw.shard_bounds(3001, r, 8, "ceil") for r in range(8)]
+    for parts in (floor, ceil):
+        assert parts[0][0] == 0 and parts[-1][1] == 3001
+        assert all(parts[i][1] == parts[i + 1][0] for i in range(7))
+    assert floor[-1][1] - floor[-1][0] == 376 and ceil[-1][1] - ceil[-1][0] == 369
+    assert tw.shard_bounds(5, 7, 8, "ceil") == (5, 5)
+
+
+def test_split_size_formula():
+    # ((N + 255) & ~255) // 2 + split_offset, vllm/model_executor/models/llama.py:521
+    assert tw.tokenweave_split_size(4096) == 2048
+    assert tw.tokenweave_split_size(4097) == 2176
+    assert tw.tokenweave_split_size(1024, 256) == 768
+    assert tw.tokenweave_split_size(1) == 128
+
+
+class _Recorder(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.calls = []
+
+    def forward(self, x, residual, **kw):
+        self.calls.append((x, residual, kw))
+
+
+def test_fused_allreduce_layernorm_slices_and_offsets_like_the_reference():
+    # tokenweave_utils.py:59-91
+    H, T, ws = 64, 32, 8
+    hs = torch.zeros(T, H, dtype=torch.bfloat16)
+    res = torch.zeros(T, H, dtype=torch.bfloat16)
+    rec = _Recorder()
+    tw.fused_allreduce_layernorm(rec, hs, res, "hdl", T // ws, 3, ws, 16, offset_symm_mem=4096)
+    x, r, kw = rec.calls[0]
+    assert x.data_ptr() == hs[12:16].data_ptr() and x.shape == (4, H)
+    assert r.data_ptr() == res[12:16].data_ptr()
+    assert kw == dict(MAX_CTAS=4, fused_ar=True, symm_mem_hdl="hdl", rank=3, world_size=ws,
+                      offset=4096 + 12 * H * 2)
+    with pytest.raises(AssertionError, match="same shape"):
+        tw.fused_allreduce_layernorm(rec, hs, res[:8], "hdl", 4, 0, ws, 16)
+    with pytest.raises(AssertionError, match="Mismatch in token count: expected 40, got 32"):
+        tw.fused_allreduce_layernorm(rec, hs, res, "hdl", 5, 0, ws, 16)
+    with pytest.raises(AssertionError, match="Invalid rank 8"):
+        tw.fused_allreduce_layernorm(rec, hs, res, "hdl", 4, 8, ws, 16)
+    # ragged extension
+    tw.fused_allreduce_layernorm(rec, hs, res, "hdl", 0, 7, ws, 16, row_range=(28, 32))
+    assert rec.calls[-1][2]["offset"] == 28 * H * 2 and rec.calls[-1][0].shape == (4, H)
+
+
+def test_rmsnorm_module_surface_and_native_path():
+    layer = tw.RMSNorm(64, eps=1e-5)
+    assert layer.weight.shape == (64,) and layer.variance_epsilon == 1e-5
+    x = torch.randn(3, 64)
+    r = torch.randn(3, 64)
+    y, r2 = layer.forward_native(x, r)
+    s = x + r
+    torch.testing.assert_close(r2, s)
+    torch.testing.assert_close(y, s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + 1e-5))
+    with pytest.raises(ValueError, match="Expected hidden_size to be 64"):
+        layer.forward_native(torch.randn(3, 32))
+    import inspect
+    params = list(inspect.signature(layer.forward).parameters)
+    assert params == ["x", "residual", "out", "MAX_CTAS", "fused_ar", "fused_rs", "symm_mem_hdl",
+                      "rank", "world_size", "offset"]
+
+
+def test_partials_region_lookup():
+    class Owner:
+        pass
+    o = Owner()
+    ops.register_partials_region(0x10000, 0x1000, 8, o)
+    assert ops._peer_stride(0x10000 + 0x800, 8) == 0x1000
+    with pytest.raises(RuntimeError, match="not inside slot 0"):
+        ops._peer_stride(0x10000 + 0x1000, 8)
+    with pytest.raises(RuntimeError, match="exceeds the 8 slots"):
+        ops._peer_stride(0x10000, 9)
+    assert ops._peer_stride(0xdead0, 1) == 16
+    del o
+    with pytest.raises(RuntimeError, match="not inside slot 0"):
+        ops._peer_stride(0x10000, 8)
+
+
+def test_algorithmic_bytes_table():
+    assert wl.algorithmic_bytes(1, 512, 8192) == 33570816
+    assert wl.algorithmic_bytes(8, 256, 8192) == 46153728
+    assert wl.algorithmic_bytes(8, 1, 8192) == 196608
+    assert wl.algorithmic_bytes(8, 3001, 8192) == 540868608
+    assert wl.algorithmic_bytes(8, 8192, 6144) == 1107308544
+    assert wl.algorithmic_bytes(8, 1638, 8192) == 295223296
+    cfgs = wl.norm_configs()
+    assert cfgs["c2_llama70b_tp8_shard@T256"].bytes == 46153728
+    assert {"c1_add_rmsnorm", "c3_qwen72b_ragged", "c4_mixtral_8x22b_chunk", "c5_weave_norm_split"} <= set(cfgs)
+
+
+def test_workload_generation_is_seeded_and_shaped():
+    cfg = wl.C3.with_tokens(5)
+    a, b = wl.make_norm_inputs(cfg, "cpu"), wl.make_norm_inputs(cfg, "cpu")
+    assert torch.equal(a.staging, b.staging) and torch.equal(a.weight, b.weight)
+    assert a.staging.shape == (8, 5, 8192) and a.residual.dtype == torch.bfloat16
+    assert 0.5 <= a.weight.float().min() and a.weight.float().max() <= 1.5
+    c = wl.make_norm_inputs(cfg, "cpu", seed_offset=1)
+    assert not torch.equal(a.staging, c.staging)
+    g = wl.make_gemm_inputs(16, 32, 64, "cpu")
+    assert g.a.shape == (16, 64) and g.b.shape == (32, 64) and abs(g.b.float().std() - 0.02) < 0.005

@@ -1,0 +1,15 @@
+"""tokenweave_amd: MI355X-native fused P-partial reduce + residual-add + RMSNorm.
+
+Python host side over the C ABI in ``include/tokenweave_amd.h``; mirrors the
+reference's op shims (``vllm/_custom_ops.py:176-221``), its ``RMSNorm`` layer
+(``vllm/model_executor/layers/layernorm.py``) and
+``fused_allreduce_layernorm`` (``vllm/model_executor/models/tokenweave_utils.py:24-92``).
+"""
+from . import _custom_ops as ops  # noqa: F401
+from .layernorm import RMSNorm  # noqa: F401
+from .tokenweave_utils import (PartialsBuffer, fused_allreduce_layernorm,  # noqa: F401
+                               shard_bounds, tokenweave_split_size, weave_norm_gemm)
+
+__all__ = ["ops", "RMSNorm", "PartialsBuffer", "fused_allreduce_layernorm", "shard_bounds",
+           "tokenweave_split_size", "weave_norm_gemm"]
+__version__ = "0.1.0"

@@ -1,0 +1,337 @@
+"""Op shims with the reference's names and argument lists.
+
+Mirror of ``vllm/_custom_ops.py:176-221``: every function mutates its tensor
+arguments in place and returns ``None``.  The same schema strings the reference
+registers in ``csrc/torch_bindings.cpp:133-171`` are registered here under the
+``tokenweave_amd`` namespace, so ``torch.ops.tokenweave_amd.fused_add_rms_norm``
+is callable exactly like ``torch.ops._C.fused_add_rms_norm``.
+
+Each op validates on the host what the HIP kernel assumes (device, dtype, row
+contiguity, shapes) and then enqueues one kernel on the current torch stream of
+the tensor's device through the C ABI.  There is no CPU implementation: calling
+an op with CPU tensors, or without the built library, raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import weakref
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.bfloat16: _lib.TW_DTYPE_BF16, torch.float16: _lib.TW_DTYPE_F16,
+               torch.float32: _lib.TW_DTYPE_F32}
+
+# Message of the reference's launchers (csrc/tokenweave_fused_kernels.cu:259).
+ALIGNMENT_MESSAGE = ("Input, residual, and weight tensors must be 16-byte aligned and "
+                     "hidden_size must be divisible by 8 for optimized kernel.")
+
+
+# ---------------------------------------------------------------------------
+# host-side checks
+# ---------------------------------------------------------------------------
+def _rows(t: torch.Tensor) -> Tuple[int, int]:
+    """(num_tokens, hidden_size) as the reference computes them
+    (csrc/layernorm_kernels.cu:198-199)."""
+    if t.dim() < 1:
+        raise RuntimeError("expected a tensor with at least one dimension")
+    hidden = t.size(-1)
+    return (t.numel() // hidden if hidden else 0), hidden
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _check_tensor(name: str, t: torch.Tensor, dtype: torch.dtype, device: torch.device) -> None:
+    _require(isinstance(t, torch.Tensor), f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"{name} is on {t.device}: tokenweave_amd ops run on the GPU only "
+            "(there is no CPU implementation)")
+    _require(t.device == device, f"{name} is on {t.device}, expected {device}")
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name} has dtype {t.dtype}, expected {dtype}")
+    _require(t.is_contiguous(),
+             f"{name} must be row-contiguous (stride(-1) == 1, stride(-2) == hidden_size); "
+             f"got shape {tuple(t.shape)} stride {tuple(t.stride())}")
+
+
+def _check_weight(weight: torch.Tensor, hidden: int, dtype, device) -> None:
+    _check_tensor("weight", weight, dtype, device)
+    _require(weight.numel() == hidden,
+             f"weight has {weight.numel()} elements, expected hidden_size {hidden}")
+
+
+def _dtype_code(name: str, t: torch.Tensor) -> int:
+    code = _DTYPE_CODE.get(t.dtype)
+    if code is None:
+        # AT_DISPATCH_SWITCH wording (csrc/dispatch_utils.h:14-21)
+        raise NotImplementedError(f'"{name}" not implemented for \'{t.dtype}\'')
+    return code
+
+
+def _require_bf16(name: str, t: torch.Tensor) -> None:
+    if t.dtype != torch.bfloat16:
+        # csrc/dispatch_utils.h:23-27: the TokenWeave kernels dispatch bf16 only
+        raise NotImplementedError(f'"{name}" not implemented for \'{t.dtype}\'')
+
+
+def _stream_ptr(t: torch.Tensor) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+class _on_device:
+    """Make the tensor's device current for the duration of the launch
+    (OptionalCUDAGuard in the reference, csrc/tokenweave_fused_kernels.cu:239)."""
+
+    def __init__(self, t: torch.Tensor):
+        self.idx = t.device.index
+        self.guard = None
+
+    def __enter__(self):
+        if self.idx is not None and self.idx != torch.cuda.current_device():
+            self.guard = torch.cuda.device(self.idx)
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+
+
+def _cap(max_ctas: Optional[int]) -> int:
+    return 0 if max_ctas is None else int(max_ctas)
+
+
+# ---------------------------------------------------------------------------
+# layer norm ops (vllm/_custom_ops.py:176-182)
+# ---------------------------------------------------------------------------
+def rms_norm(out: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,
+             epsilon: float) -> None:
+    code = _dtype_code("rms_norm_kernel", input)
+    _check_tensor("input", input, input.dtype, input.device)
+    _check_tensor("out", out, input.dtype, input.device)
+    T, H = _rows(input)
+    _require(out.shape == input.shape, "out and input must have the same shape")
+    _check_weight(weight, H, input.dtype, input.device)
+    with _on_device(input):
+        _lib.check(_lib.lib().tw_rms_norm(out.data_ptr(), input.data_ptr(), weight.data_ptr(),
+                                          T, H, epsilon, code, _stream_ptr(input)))
+
+
+def fused_add_rms_norm(input: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,
+                       epsilon: float) -> None:
+    code = _dtype_code("fused_add_rms_norm_kernel", input)
+    _check_tensor("input", input, input.dtype, input.device)
+    _check_tensor("residual", residual, input.dtype, input.device)
+    T, H = _rows(input)
+    _require(residual.shape == input.shape, "input and residual must have the same shape")
+    _check_weight(weight, H, input.dtype, input.device)
+    with _on_device(input):
+        _lib.check(_lib.lib().tw_fused_add_rms_norm(
+            input.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H, epsilon, code,
+            _stream_ptr(input)))
+
+
+# ---------------------------------------------------------------------------
+# TokenWeave ops (vllm/_custom_ops.py:184-207)
+# ---------------------------------------------------------------------------
+def rms_norm_inplace(out: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,
+                     epsilon: float) -> None:
+    code = _dtype_code("rms_norm_inplace_kernel", input)
+    _check_tensor("input", input, input.dtype, input.device)
+    _check_tensor("out", out, input.dtype, input.device)
+    T, H = _rows(input)
+    _require(out.shape == input.shape, "out and input must have the same shape")
+    _check_weight(weight, H, input.dtype, input.device)
+    with _on_device(input):
+        _lib.check(_lib.lib().tw_rms_norm_inplace(
+            out.data_ptr(), input.data_ptr(), weight.data_ptr(), T, H, epsilon, code,
+            _stream_ptr(input)))
+
+
+def fused_add_rms_norm_cta(input: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,
+                           MAX_CTAS: int, epsilon: float) -> None:
+    _require_bf16("fused_add_rms_norm_cta_kernel", input)
+    _check_tensor("input", input, torch.bfloat16, input.device)
+    _check_tensor("residual", residual, torch.bfloat16, input.device)
+    T, H = _rows(input)
+    _require(residual.shape == input.shape, "input and residual must have the same shape")
+    _check_weight(weight, H, torch.bfloat16, input.device)
+    with _on_device(input):
+        _lib.check(_lib.lib().tw_fused_add_rms_norm_cta(
+            input.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H, _cap(MAX_CTAS),
+            epsilon, _stream_ptr(input)))
+
+
+# --- one-GPU stand-in for the symmetric-memory address space -----------------
+# The reference passes `mcptr`, one multicast address that names the same offset
+# in every rank's staging buffer (layernorm.py:79).  On one GPU the P staging
+# buffers are slots of one allocation; a registered region tells the shim the
+# distance between slots so that `mcptr + p * stride` is partial p.
+_REGIONS: List[Tuple[int, int, int, "weakref.ref"]] = []  # (base, stride_bytes, slots, owner)
+
+
+def register_partials_region(base_ptr: int, stride_bytes: int, slots: int, owner) -> None:
+    """Declare [base_ptr, base_ptr + slots*stride_bytes) as `slots` equally spaced
+    partial-sum buffers.  `owner` is weakly referenced; the region is dropped with it."""
+    _require(stride_bytes > 0 and stride_bytes % 16 == 0, "slot stride must be a positive multiple of 16")
+    _require(1 <= slots <= _lib.TW_MAX_PARTIALS, f"slots must be in [1, {_lib.TW_MAX_PARTIALS}]")
+    _prune_regions()
+    _REGIONS.append((int(base_ptr), int(stride_bytes), int(slots), weakref.ref(owner)))
+
+
+def _prune_regions() -> None:
+    _REGIONS[:] = [r for r in _REGIONS if r[3]() is not None]
+
+
+def _peer_stride(mcptr: int, world_size: int) -> int:
+    if world_size == 1:
+        return 16  # unused: there is only partial 0
+    _prune_regions()
+    for base, stride, slots, _ in _REGIONS:
+        if base <= mcptr < base + stride:
+            _require(world_size <= slots,
+                     f"world_size {world_size} exceeds the {slots} slots of the partials region")
+            return stride
+    raise RuntimeError(
+        f"mcptr 0x{mcptr:x} is not inside slot 0 of a registered partials region "
+        "(allocate the staging buffers with tokenweave_amd.PartialsBuffer)")
+
+
+def _fused_rs_ln(entry: str, kname: str, input, residual, weight, mcptr, signal_pads, rank,
+                 world_size, MAX_CTAS, epsilon) -> None:
+    del signal_pads  # no peers, no signal pads on one GPU
+    _require_bf16(kname, input)
+    _check_tensor("input", input, torch.bfloat16, input.device)
+    _check_tensor("residual", residual, torch.bfloat16, input.device)
+    T, H = _rows(input)
+    _require(residual.shape == input.shape, "input and residual must have the same shape")
+    _check_weight(weight, H, torch.bfloat16, input.device)
+    _require(0 <= rank < world_size, f"Invalid rank {rank}, must be in [0, {world_size - 1}]")
+    stride = _peer_stride(int(mcptr), int(world_size))
+    with _on_device(input):
+        _lib.check(getattr(_lib.lib(), entry)(
+            input.data_ptr(), residual.data_ptr(), weight.data_ptr(), int(mcptr), stride,
+            int(rank), int(world_size), _cap(MAX_CTAS), epsilon, T, H, _stream_ptr(input)))
+
+
+def fused_rs_ln_ag_cta(input: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,
+                       mcptr: int, signal_pads: int, rank: int, world_size: int, MAX_CTAS: int,
+                       epsilon: float) -> None:
+    _fused_rs_ln("tw_fused_rs_ln_ag_cta", "fused_rs_ln_ag_cta_kernel", input, residual, weight,
+                 mcptr, signal_pads, rank, world_size, MAX_CTAS, epsilon)
+
+
+def fused_rs_ln_cta(input: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,
+                    mcptr: int, signal_pads: int, rank: int, world_size: int, MAX_CTAS: int,
+                    epsilon: float) -> None:
+    _fused_rs_ln("tw_fused_rs_ln_cta", "fused_rs_ln_cta_kernel", input, residual, weight,
+                 mcptr, signal_pads, rank, world_size, MAX_CTAS, epsilon)
+
+
+# ---------------------------------------------------------------------------
+# one-GPU general form and the weave GEMM (no counterpart in vllm/_custom_ops.py)
+# ---------------------------------------------------------------------------
+def reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
+                        residual: torch.Tensor, weight: torch.Tensor, epsilon: float,
+                        MAX_CTAS: Optional[int] = None) -> None:
+    """out <- RMSNorm(sum_p partials[p] + residual) * weight; residual <- the sum.
+    `out` may be one of the partials."""
+    P = len(partials)
+    _require(1 <= P <= _lib.TW_MAX_PARTIALS,
+             f"number of partials {P} not in [1, {_lib.TW_MAX_PARTIALS}]")
+    _require_bf16("reduce_add_rms_norm_kernel", out)
+    dev = out.device
+    _check_tensor("out", out, torch.bfloat16, dev)
+    _check_tensor("residual", residual, torch.bfloat16, dev)
+    T, H = _rows(out)
+    _require(residual.shape == out.shape, "out and residual must have the same shape")
+    for i, p in enumerate(partials):
+        _check_tensor(f"partials[{i}]", p, torch.bfloat16, dev)
+        _require(p.shape == out.shape, f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(out.shape)}")
+    _check_weight(weight, H, torch.bfloat16, dev)
+    ptrs = (ctypes.c_void_p * P)(*[p.data_ptr() for p in partials])
+    with _on_device(out):
+        _lib.check(_lib.lib().tw_reduce_add_rms_norm(
+            ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H,
+            _cap(MAX_CTAS), epsilon, _stream_ptr(out)))
+
+
+def gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
+                 max_cus: Optional[int] = None) -> None:
+    """out[M, N] <- a[M, K] @ b[N, K]^T (bf16, fp32 accumulate).  `out` may be a row
+    slice of a wider buffer (row stride >= N).  The in-place row-parallel linear of
+    vllm/model_executor/layers/linear.py:203-228."""
+    _require_bf16("gemm_bf16_nt_kernel", a)
+    dev = a.device
+    _check_tensor("a", a, torch.bfloat16, dev)
+    _check_tensor("b", b, torch.bfloat16, dev)
+    _require(a.dim() == 2 and b.dim() == 2 and out.dim() == 2, "gemm operands must be 2-D")
+    _require(out.is_cuda and out.device == dev and out.dtype == torch.bfloat16,
+             "out must be a bf16 tensor on the same device")
+    M, K = a.shape
+    N, K2 = b.shape
+    _require(K == K2, f"inner dimensions differ: a is {tuple(a.shape)}, b is {tuple(b.shape)}")
+    _require(tuple(out.shape) == (M, N), f"out has shape {tuple(out.shape)}, expected {(M, N)}")
+    _require(out.stride(1) == 1 and (M <= 1 or out.stride(0) >= N), "out rows must be contiguous")
+    ldc = out.stride(0) if M > 1 else max(N, out.stride(0))
+    with _on_device(a):
+        _lib.check(_lib.lib().tw_gemm_bf16_nt(out.data_ptr(), a.data_ptr(), b.data_ptr(), M, N, K,
+                                              ldc, _cap(max_cus), _stream_ptr(a)))
+
+
+def num_compute_units(device=None) -> int:
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    with torch.cuda.device(dev):
+        n = _lib.lib().tw_num_compute_units()
+    _require(n > 0, "could not query the device's compute-unit count")
+    return n
+
+
+# ---------------------------------------------------------------------------
+# torch.library registration: the reference's schema strings
+# (csrc/torch_bindings.cpp:135-171), namespace `tokenweave_amd`.
+# ---------------------------------------------------------------------------
+SCHEMAS = {
+    "rms_norm": "rms_norm(Tensor! result, Tensor input, Tensor weight, float epsilon) -> ()",
+    "fused_add_rms_norm":
+        "fused_add_rms_norm(Tensor! input, Tensor! residual, Tensor weight, float epsilon) -> ()",
+    "rms_norm_inplace":
+        "rms_norm_inplace(Tensor! result, Tensor! input, Tensor weight, float epsilon) -> ()",
+    "fused_rs_ln_ag_cta":
+        "fused_rs_ln_ag_cta(Tensor! input, Tensor! residual, Tensor weight, int mcptr, "
+        "int signal_pads, int rank, int world_size, int MAX_CTAS, float epsilon) -> ()",
+    "fused_add_rms_norm_cta":
+        "fused_add_rms_norm_cta(Tensor! input, Tensor! residual, Tensor weight, int MAX_CTAS, "
+        "float epsilon) -> ()",
+    "fused_rs_ln_cta":
+        "fused_rs_ln_cta(Tensor! input, Tensor! residual, Tensor weight, int mcptr, "
+        "int signal_pads, int rank, int world_size, int MAX_CTAS, float epsilon) -> ()",
+}
+
+_IMPLS = {
+    "rms_norm": rms_norm,
+    "fused_add_rms_norm": fused_add_rms_norm,
+    "rms_norm_inplace": rms_norm_inplace,
+    "fused_rs_ln_ag_cta": fused_rs_ln_ag_cta,
+    "fused_add_rms_norm_cta": fused_add_rms_norm_cta,
+    "fused_rs_ln_cta": fused_rs_ln_cta,
+}
+
+
+def _no_cpu(name):
+    def impl(*args, **kwargs):
+        raise RuntimeError(f"tokenweave_amd::{name} has no CPU implementation; "
+                           "pass tensors that live on the MI355X")
+    return impl
+
+
+_library = torch.library.Library("tokenweave_amd", "DEF")
+for _name, _schema in SCHEMAS.items():
+    _library.define(_schema)
+    _library.impl(_name, _IMPLS[_name], "CUDA")
+    _library.impl(_name, _no_cpu(_name), "CPU")

@@ -1,0 +1,405 @@
+// Fused P-partial reduce + residual-add + RMSNorm for gfx950 (MI355X, wave64).
+//
+// One workgroup owns one token row at a time.  For hidden sizes up to 8192 each
+// lane owns exactly one 16-byte vector (8 bf16) of the row in every buffer: it
+// issues the P partial loads, the residual load and the weight load back to
+// back, so a 1024-lane workgroup keeps (P+1)*16 KiB of HBM reads in flight, and
+// the whole row stays in registers between the sum-of-squares reduction and the
+// normalised store — nothing is read twice.  Rows are walked with stride
+// gridDim.x, so the same kernel serves the one-row-per-workgroup launch and the
+// capped ("persistent CTA") launch.
+//
+// What this replaces in the reference: fused_rs_ln_ag_cta_kernel
+// (csrc/tokenweave_fused_kernels.cu:80-155), fused_rs_ln_cta_kernel and
+// fused_add_rms_norm_cta_kernel (csrc/tokenweave_artifact_kernels.cu:129-204,
+// :38-104), fused_add_rms_norm_kernel / rms_norm_kernel
+// (csrc/layernorm_kernels.cu:62-158, :22-54) and rms_norm_inplace_kernel
+// (csrc/tokenweave_fused_kernels.cu:37-72).  Arithmetic follows the reference's
+// CPU path (csrc/cpu/layernorm.cpp:44-88): fp32 sum, sum of squares of the
+// unrounded sum, output computed from the rounded residual with one rounding.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tw_common.h"
+
+namespace tw {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+struct PartialPtrs {
+  const void* p[TW_MAX_PARTIALS];
+};
+
+// ---------------------------------------------------------------------------
+// bf16 helpers.  A 32-bit word holds two bf16: element 2i in the low half.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+
+// Round-to-nearest-even pack (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+__device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
+  f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x);
+  f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+  f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z);
+  f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+}
+
+__device__ __forceinline__ void add8(const uint4& v, float (&f)[8]) {
+  f[0] += bf16_lo(v.x); f[1] += bf16_hi(v.x);
+  f[2] += bf16_lo(v.y); f[3] += bf16_hi(v.y);
+  f[4] += bf16_lo(v.z); f[5] += bf16_hi(v.z);
+  f[6] += bf16_lo(v.w); f[7] += bf16_hi(v.w);
+}
+
+// ---------------------------------------------------------------------------
+// Sum over the workgroup, result in every lane.  Fixed order, so a row's sum
+// depends only on the row's data and on blockDim.x.
+//   lanes:  xor-1, xor-2 (quad permutes), half-row mirror, row mirror on DPP —
+//           every lane of a 16-lane row then holds that row's sum;
+//   rows:   ((row0 + row1) + row2) + row3 through v_readlane;
+//   waves:  one LDS slot per wave, one barrier, every lane adds the slots in
+//           wave order (broadcast reads).
+// `slots` must hold 16 floats and must not be reused before the next barrier
+// (callers alternate between two slot arrays).
+// ---------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true);
+  return v + __int_as_float(moved);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+  v = dpp_add<0xB1>(v);   // quad_perm:[1,0,3,2]
+  v = dpp_add<0x4E>(v);   // quad_perm:[2,3,0,1]
+  v = dpp_add<0x141>(v);  // row_half_mirror
+  v = dpp_add<0x140>(v);  // row_mirror
+  float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return ((r0 + r1) + r2) + r3;
+}
+
+__device__ __forceinline__ float block_sum(float v, float* slots, int nwaves) {
+  v = wave_sum(v);
+  if (nwaves == 1) return v;
+  if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float total = slots[0];
+  for (int i = 1; i < nwaves; ++i) total += slots[i];
+  return total;
+}
+
+__device__ __forceinline__ float inv_rms(float ss, float hidden, float eps) {
+  // Same expression as csrc/cpu/layernorm.cpp:72-73; hipcc keeps fp32 division
+  // and sqrt correctly rounded.
+  return 1.0f / sqrtf(ss / hidden + eps);
+}
+
+// ---------------------------------------------------------------------------
+// Vector kernel, bf16.
+//   NP       number of partial buffers known at compile time, 0 = use np_rt
+//   VPT      16-byte vectors per lane per buffer (row length <= VPT*blockDim*8)
+//   HAS_RES  add the residual and write the rounded sum back to it
+//   COPY     also store the untouched first partial to `copy_out`
+//            (rms_norm_inplace: the copy becomes the residual stream)
+// y may alias any partial: a lane stores y only to vector slots it has already
+// read in every buffer.
+// ---------------------------------------------------------------------------
+template <int NP, int VPT, bool HAS_RES, bool COPY>
+__global__ __launch_bounds__(1024) void row_norm_bf16_kernel(
+    PartialPtrs parts, int np_rt, uint4* y_out, uint4* residual, uint4* copy_out,
+    const uint4* __restrict__ weight, float eps, int num_tokens, int vec_per_row,
+    float hidden) {
+  __shared__ float slots[2][16];
+  const int tid = threadIdx.x;
+  const int nt = blockDim.x;
+  const int nwaves = nt >> 6;
+  const int np = NP > 0 ? NP : np_rt;
+
+  uint4 wv[VPT];
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int v = tid + k * nt;
+    wv[k] = v < vec_per_row ? weight[v] : make_uint4(0, 0, 0, 0);
+  }
+
+  int phase = 0;
+  for (int row = blockIdx.x; row < num_tokens; row += gridDim.x, phase ^= 1) {
+    const size_t base = (size_t)row * vec_per_row;
+    float s[VPT][8];
+    float ss = 0.0f;
+
+    if (NP > 0) {
+      // Issue every load of the row before the first use.
+      uint4 a[VPT][NP > 0 ? NP : 1];
+      uint4 rv[VPT];
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        const int v = tid + k * nt;
+        if (v < vec_per_row) {
+#pragma unroll
+          for (int p = 0; p < NP; ++p)
+            a[k][p] = static_cast<const uint4*>(parts.p[p])[base + v];
+          if (HAS_RES) rv[k] = residual[base + v];
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        const int v = tid + k * nt;
+        if (v < vec_per_row) {
+          unpack8(a[k][0], s[k]);
+#pragma unroll
+          for (int p = 1; p < NP; ++p) add8(a[k][p], s[k]);
+          if (HAS_RES) add8(rv[k], s[k]);
+          if (COPY) copy_out[base + v] = a[k][0];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        const int v = tid + k * nt;
+        if (v < vec_per_row) {
+          uint4 first = static_cast<const uint4*>(parts.p[0])[base + v];
+          unpack8(first, s[k]);
+          for (int p = 1; p < np; ++p)
+            add8(static_cast<const uint4*>(parts.p[p])[base + v], s[k]);
+          if (HAS_RES) add8(residual[base + v], s[k]);
+          if (COPY) copy_out[base + v] = first;
+        }
+      }
+    }
+
+    // Sum of squares of the unrounded fp32 sum; round the residual once.
+    uint4 rnew[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int v = tid + k * nt;
+      if (v < vec_per_row) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += s[k][e] * s[k][e];
+        rnew[k].x = pack_bf16(s[k][0], s[k][1]);
+        rnew[k].y = pack_bf16(s[k][2], s[k][3]);
+        rnew[k].z = pack_bf16(s[k][4], s[k][5]);
+        rnew[k].w = pack_bf16(s[k][6], s[k][7]);
+        if (HAS_RES) residual[base + v] = rnew[k];
+      }
+    }
+
+    const float total = block_sum(ss, slots[phase], nwaves);
+    const float inv = inv_rms(total, hidden, eps);
+
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int v = tid + k * nt;
+      if (v < vec_per_row) {
+        float r[8], w[8];
+        unpack8(rnew[k], r);
+        unpack8(wv[k], w);
+        uint4 o;
+        o.x = pack_bf16(r[0] * inv * w[0], r[1] * inv * w[1]);
+        o.y = pack_bf16(r[2] * inv * w[2], r[3] * inv * w[3]);
+        o.z = pack_bf16(r[4] * inv * w[4], r[5] * inv * w[5]);
+        o.w = pack_bf16(r[6] * inv * w[6], r[7] * inv * w[7]);
+        y_out[base + v] = o;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Element-wise kernel: any hidden size, any alignment, bf16 / fp16 / fp32.
+// Two passes over the row; the second re-reads the rounded residual (or the
+// input when there is none), like the reference's generic kernel
+// (csrc/layernorm_kernels.cu:122-158).
+// ---------------------------------------------------------------------------
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+  static __device__ __forceinline__ float load(const __bf16* p) {
+    return __uint_as_float((uint32_t)(*reinterpret_cast<const uint16_t*>(p)) << 16);
+  }
+  static __device__ __forceinline__ __bf16 round(float f) { return (__bf16)f; }
+};
+template <> struct Elem<_Float16> {
+  static __device__ __forceinline__ float load(const _Float16* p) { return (float)*p; }
+  static __device__ __forceinline__ _Float16 round(float f) { return (_Float16)f; }
+};
+template <> struct Elem<float> {
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ float round(float f) { return f; }
+};
+
+template <typename T, bool HAS_RES, bool COPY>
+__global__ __launch_bounds__(1024) void row_norm_elem_kernel(
+    PartialPtrs parts, int np, T* y_out, T* residual, T* copy_out,
+    const T* __restrict__ weight, float eps, int num_tokens, int hidden_size) {
+  __shared__ float slots[2][16];
+  const int tid = threadIdx.x;
+  const int nt = blockDim.x;
+  const int nwaves = nt >> 6;
+  int phase = 0;
+  for (int row = blockIdx.x; row < num_tokens; row += gridDim.x, phase ^= 1) {
+    const size_t base = (size_t)row * hidden_size;
+    float ss = 0.0f;
+    for (int j = tid; j < hidden_size; j += nt) {
+      float s = Elem<T>::load(static_cast<const T*>(parts.p[0]) + base + j);
+      for (int p = 1; p < np; ++p)
+        s += Elem<T>::load(static_cast<const T*>(parts.p[p]) + base + j);
+      if (HAS_RES) {
+        s += Elem<T>::load(residual + base + j);
+        residual[base + j] = Elem<T>::round(s);
+      }
+      ss += s * s;
+    }
+    const float total = block_sum(ss, slots[phase], nwaves);
+    const float inv = inv_rms(total, (float)hidden_size, eps);
+    const T* src = HAS_RES ? residual : static_cast<const T*>(parts.p[0]);
+    for (int j = tid; j < hidden_size; j += nt) {
+      const T raw = src[base + j];
+      const float r = Elem<T>::load(&raw);
+      if (COPY) copy_out[base + j] = raw;
+      y_out[base + j] = Elem<T>::round(r * inv * Elem<T>::load(weight + j));
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+static int default_grid(int64_t num_tokens) {
+  // One workgroup per row until the rows outnumber what the device keeps
+  // resident (two 1024-lane workgroups per compute unit); beyond that the
+  // resident workgroups walk the rows.
+  const int cus = device_compute_units();
+  const int64_t resident = (int64_t)(cus > 0 ? cus : 256) * 2;
+  return (int)(num_tokens < resident ? num_tokens : resident);
+}
+
+template <int NP, bool HAS_RES, bool COPY>
+static int launch_vec_vpt(const PartialPtrs& parts, int np, void* y, void* residual,
+                          void* copy_out, const void* weight, int64_t T, int64_t H,
+                          float eps, int grid, hipStream_t stream) {
+  const int V = (int)(H / 8);
+  int nt = V < 1024 ? ((V + 63) / 64) * 64 : 1024;
+  const int vpt = (V + nt - 1) / nt;
+  dim3 g(grid), b(nt);
+#define TW_LAUNCH(VPT)                                                              \
+  hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, HAS_RES, COPY>), g, b, 0, stream, \
+                     parts, np, static_cast<uint4*>(y), static_cast<uint4*>(residual), \
+                     static_cast<uint4*>(copy_out), static_cast<const uint4*>(weight), \
+                     eps, (int)T, V, (float)H)
+  if (vpt == 1) TW_LAUNCH(1);
+  else if (vpt == 2) TW_LAUNCH(2);
+  else if (vpt <= 4) TW_LAUNCH(4);
+  else return 1;  // caller falls back to the element-wise kernel
+#undef TW_LAUNCH
+  return 0;
+}
+
+template <typename T>
+static void launch_elem_t(const PartialPtrs& parts, int np, void* y, void* residual,
+                          void* copy_out, const void* weight, int64_t Tn, int64_t H,
+                          float eps, int grid, hipStream_t stream) {
+  int nt = H < 1024 ? (int)((H + 63) / 64) * 64 : 1024;
+  dim3 g(grid), b(nt);
+#define TW_LAUNCH(HAS_RES, COPY)                                                     \
+  hipLaunchKernelGGL((row_norm_elem_kernel<T, HAS_RES, COPY>), g, b, 0, stream, parts, \
+                     np, static_cast<T*>(y), static_cast<T*>(residual),               \
+                     static_cast<T*>(copy_out), static_cast<const T*>(weight), eps,   \
+                     (int)Tn, (int)H)
+  if (residual) TW_LAUNCH(true, false);
+  else if (copy_out) TW_LAUNCH(false, true);
+  else TW_LAUNCH(false, false);
+#undef TW_LAUNCH
+}
+
+static int finish_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return set_error(TW_ERR_LAUNCH, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
+  return TW_OK;
+}
+
+// Shared by every entry point.  residual == nullptr: no residual add;
+// copy_out != nullptr: rms_norm_inplace.  require_vec: refuse instead of
+// falling back to the element-wise kernel (the *_cta contract).
+int run_row_norm(const char* what, const void* const* partials, int np, void* y,
+                 void* residual, void* copy_out, const void* weight, int64_t T,
+                 int64_t H, float eps, int dtype, int max_ctas, bool require_vec,
+                 void* stream_v) {
+  if (np < 1 || np > TW_MAX_PARTIALS)
+    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: number of partials %d not in [1, %d]", what, np,
+                     TW_MAX_PARTIALS);
+  if (T < 0 || H <= 0 || T > INT32_MAX || H > INT32_MAX)
+    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: bad shape num_tokens=%lld hidden_size=%lld", what,
+                     (long long)T, (long long)H);
+  if (dtype != TW_DTYPE_BF16 && dtype != TW_DTYPE_F16 && dtype != TW_DTYPE_F32)
+    return set_error(TW_ERR_DTYPE, "%s: unknown dtype code %d", what, dtype);
+  if (T == 0) return TW_OK;
+  if (!y || !weight || !partials)
+    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: null pointer argument", what);
+  PartialPtrs parts = {};
+  bool aligned = aligned16(y) && aligned16(weight) && (!residual || aligned16(residual)) &&
+                 (!copy_out || aligned16(copy_out));
+  for (int p = 0; p < np; ++p) {
+    if (!partials[p])
+      return set_error(TW_ERR_INVALID_ARGUMENT, "%s: partial %d is a null pointer", what, p);
+    parts.p[p] = partials[p];
+    aligned = aligned && aligned16(partials[p]);
+  }
+  const bool vec_ok = aligned && (H % 8 == 0);
+  if (require_vec && (!vec_ok || dtype != TW_DTYPE_BF16)) {
+    if (dtype != TW_DTYPE_BF16)
+      return set_error(TW_ERR_DTYPE, "%s: only bf16 is supported", what);
+    // Message of the reference's launcher (csrc/tokenweave_fused_kernels.cu:259).
+    return set_error(TW_ERR_ALIGNMENT,
+                     "Input, residual, and weight tensors must be 16-byte aligned and "
+                     "hidden_size must be divisible by 8 for optimized kernel.");
+  }
+  int grid = max_ctas > 0 ? max_ctas : default_grid(T);
+  if (grid > T) grid = (int)T;
+  hipStream_t stream = static_cast<hipStream_t>(stream_v);
+
+  if (vec_ok && dtype == TW_DTYPE_BF16) {
+    int fell = 1;
+#define TW_MODE(NP)                                                                       \
+  (residual ? launch_vec_vpt<NP, true, false>(parts, np, y, residual, nullptr, weight, T, \
+                                              H, eps, grid, stream)                       \
+   : copy_out ? launch_vec_vpt<NP, false, true>(parts, np, y, nullptr, copy_out, weight,  \
+                                                T, H, eps, grid, stream)                  \
+              : launch_vec_vpt<NP, false, false>(parts, np, y, nullptr, nullptr, weight,  \
+                                                 T, H, eps, grid, stream))
+    switch (np) {
+      case 1: fell = TW_MODE(1); break;
+      case 2: fell = residual ? launch_vec_vpt<2, true, false>(parts, np, y, residual, nullptr, weight, T, H, eps, grid, stream) : 1; break;
+      case 4: fell = residual ? launch_vec_vpt<4, true, false>(parts, np, y, residual, nullptr, weight, T, H, eps, grid, stream) : 1; break;
+      case 8: fell = residual ? launch_vec_vpt<8, true, false>(parts, np, y, residual, nullptr, weight, T, H, eps, grid, stream) : 1; break;
+      default: fell = residual ? launch_vec_vpt<0, true, false>(parts, np, y, residual, nullptr, weight, T, H, eps, grid, stream) : 1; break;
+    }
+#undef TW_MODE
+    if (fell == 0) return finish_launch(what);
+    // rows longer than 4 vectors per lane: the element-wise kernel below
+  }
+  switch (dtype) {
+    case TW_DTYPE_BF16:
+      launch_elem_t<__bf16>(parts, np, y, residual, copy_out, weight, T, H, eps, grid, stream);
+      break;
+    case TW_DTYPE_F16:
+      launch_elem_t<_Float16>(parts, np, y, residual, copy_out, weight, T, H, eps, grid, stream);
+      break;
+    default:
+      launch_elem_t<float>(parts, np, y, residual, copy_out, weight, T, H, eps, grid, stream);
+      break;
+  }
+  return finish_launch(what);
+}
+
+}  // namespace tw

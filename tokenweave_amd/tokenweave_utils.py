@@ -1,0 +1,161 @@
+"""Host-side orchestration of the fused op: row sharding, the staging buffers
+that stand in for symmetric memory on one GPU, and the two-stream weave step.
+
+Mirror of ``vllm/model_executor/models/tokenweave_utils.py``:
+``fused_allreduce_layernorm`` (:24-92) keeps its argument list, assertions and
+slice/offset arithmetic; ``weave_norm_gemm`` is one stage of
+``tokenweave_overlap`` (:236-260) — the norm of one token split on a second
+stream while the other split's row-parallel GEMM runs on the current stream.
+"""
+from __future__ import annotations
+
+from typing import Any, Callable, Optional, Tuple
+
+import torch
+
+from . import _custom_ops as ops
+from .layernorm import RMSNorm
+
+
+class PartialsBuffer:
+    """The P ranks' staging buffers as P equally spaced slots of one allocation.
+
+    In the reference every rank owns one symmetric-memory staging buffer and
+    ``symm_mem_hdl.multicast_ptr`` names all of them at once
+    (vllm/model_executor/models/llama.py:437-441).  Here slot p holds what rank
+    p's buffer would hold — its partial sum — and the object exposes the two
+    attributes the layer reads from the handle (layernorm.py:79-80):
+    ``multicast_ptr`` (address of slot 0) and ``signal_pad_ptrs_dev`` (0: there
+    are no peers to signal).  Rows are [max_tokens, hidden_size] bf16.
+    """
+
+    def __init__(self, world_size: int, max_tokens: int, hidden_size: int, rank: int = 0,
+                 device: Any = "cuda", dtype: torch.dtype = torch.bfloat16) -> None:
+        assert 0 <= rank < world_size, f"Invalid rank {rank}, must be in [0, {world_size - 1}]"
+        if dtype != torch.bfloat16:
+            raise NotImplementedError("staging buffers are bf16, like the reference's")
+        if hidden_size % 8 != 0:
+            raise RuntimeError(ops.ALIGNMENT_MESSAGE)
+        self.world_size = world_size
+        self.rank = rank
+        self.max_tokens = max_tokens
+        self.hidden_size = hidden_size
+        self.storage = torch.empty(world_size, max_tokens, hidden_size, dtype=dtype, device=device)
+        self.peer_stride_bytes = max_tokens * hidden_size * self.storage.element_size()
+        self.multicast_ptr = self.storage.data_ptr()
+        self.signal_pad_ptrs_dev = 0
+        ops.register_partials_region(self.multicast_ptr, self.peer_stride_bytes, world_size,
+                                     self.storage)
+
+    def slot(self, p: int) -> torch.Tensor:
+        """Rank p's staging buffer, [max_tokens, hidden_size]."""
+        return self.storage[p]
+
+    @property
+    def local(self) -> torch.Tensor:
+        """This rank's staging buffer: where its GEMM writes and where y lands."""
+        return self.storage[self.rank]
+
+    def hidden_states(self, num_tokens: int, first_row: int = 0) -> torch.Tensor:
+        return self.local[first_row:first_row + num_tokens]
+
+    def offset_of_row(self, row: int) -> int:
+        """Byte offset of a row inside every slot (`offset_symm_mem` of the reference)."""
+        return row * self.hidden_size * self.storage.element_size()
+
+
+def shard_bounds(total_tokens: int, rank: int, world_size: int,
+                 mode: str = "even") -> Tuple[int, int]:
+    """Rows [start, end) that `rank` owns.
+
+    "even"  — the reference's contract: total_tokens == per_rank * world_size
+              (tokenweave_utils.py:63-77);
+    "floor" — per_rank = total // world_size, the last rank takes the remainder;
+    "ceil"  — per_rank = ceil(total / world_size), the last ranks take what is left.
+    """
+    assert 0 <= rank < world_size, f"Invalid rank {rank}, must be in [0, {world_size - 1}]"
+    if mode == "even":
+        per = total_tokens // world_size
+        assert per * world_size == total_tokens, (
+            f"Mismatch in token count: expected {per * world_size}, got {total_tokens}")
+        return rank * per, (rank + 1) * per
+    if mode == "floor":
+        per = total_tokens // world_size
+        start = rank * per
+        return start, (total_tokens if rank == world_size - 1 else start + per)
+    if mode == "ceil":
+        per = -(-total_tokens // world_size)
+        start = min(rank * per, total_tokens)
+        return start, min(start + per, total_tokens)
+    raise ValueError(f"unknown shard mode {mode!r}")
+
+
+def fused_allreduce_layernorm(
+    layernorm: RMSNorm,
+    hidden_states: torch.Tensor,
+    residual: torch.Tensor,
+    symm_mem_hdl: Any,
+    num_tokens_per_rank: int,
+    rank: int,
+    world_size: int,
+    MAX_CTAS: int,
+    offset_symm_mem: int = 0,
+    row_range: Optional[Tuple[int, int]] = None,
+) -> None:
+    """Fused reduce + residual add + RMSNorm on this rank's rows, in place.
+
+    hidden_states / residual: [total_tokens, hidden] — this rank's staging rows
+    and the residual stream.  Same contract as the reference
+    (tokenweave_utils.py:24-92).  `row_range=(start, end)` overrides the even
+    split for ragged token counts (the reference pads instead, llama.py:536).
+    """
+    assert hidden_states.shape == residual.shape, \
+        "hidden_states and residual must have the same shape"
+    assert 0 <= rank < world_size, f"Invalid rank {rank}, must be in [0, {world_size - 1}]"
+    total_tokens = hidden_states.shape[0]
+    if row_range is None:
+        expected_tokens = num_tokens_per_rank * world_size
+        assert total_tokens == expected_tokens, (
+            f"Mismatch in token count: expected {expected_tokens}, got {total_tokens}")
+        start_idx = rank * num_tokens_per_rank
+        end_idx = (rank + 1) * num_tokens_per_rank
+    else:
+        start_idx, end_idx = row_range
+        assert 0 <= start_idx <= end_idx <= total_tokens, \
+            f"row_range {row_range} outside [0, {total_tokens}]"
+    rows = end_idx - start_idx
+    if rows == 0:
+        return
+    row_bytes = hidden_states.shape[1] * hidden_states.element_size()
+    layernorm(
+        hidden_states[start_idx:end_idx],
+        residual[start_idx:end_idx],
+        MAX_CTAS=min(MAX_CTAS, rows),
+        fused_ar=True,
+        symm_mem_hdl=symm_mem_hdl,
+        rank=rank,
+        world_size=world_size,
+        offset=offset_symm_mem + start_idx * row_bytes,
+    )
+
+
+def tokenweave_split_size(num_tokens: int, split_offset: int = 0) -> int:
+    """Rows of the first token split (vllm/model_executor/models/llama.py:521):
+    half of the token count rounded up to a multiple of 256, plus an offset."""
+    return ((num_tokens + 255) & ~255) // 2 + split_offset
+
+
+def weave_norm_gemm(gemm: Callable[[], None], norm: Callable[[], None],
+                    norm_stream: torch.cuda.Stream) -> None:
+    """One weave stage: `norm` (the fused reduce+norm of one token split) is
+    enqueued on `norm_stream`, `gemm` (the other split's row-parallel GEMM) on the
+    current stream, with the reference's hand-offs on both sides
+    (tokenweave_utils.py:238-260): the norm stream first waits for everything
+    already queued on the current stream, and the current stream afterwards waits
+    for the norm.  Both streams keep the default priority."""
+    current = torch.cuda.current_stream()
+    norm_stream.wait_stream(current)
+    with torch.cuda.stream(norm_stream):
+        norm()
+    gemm()
+    current.wait_stream(norm_stream)

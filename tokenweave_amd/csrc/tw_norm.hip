@@ -1,13 +1,26 @@
 // Fused P-partial reduce + residual-add + RMSNorm for gfx950 (MI355X, wave64).
 //
-// One workgroup owns one token row at a time.  For hidden sizes up to 8192 each
-// lane owns exactly one 16-byte vector (8 bf16) of the row in every buffer: it
-// issues the P partial loads, the residual load and the weight load back to
-// back, so a 1024-lane workgroup keeps (P+1)*16 KiB of HBM reads in flight, and
-// the whole row stays in registers between the sum-of-squares reduction and the
-// normalised store — nothing is read twice.  Rows are walked with stride
-// gridDim.x, so the same kernel serves the one-row-per-workgroup launch and the
-// capped ("persistent CTA") launch.
+// One workgroup owns one token row at a time and keeps the whole row in
+// registers between the sum-of-squares reduction and the normalised store:
+// every byte is read once and written once.  At hidden size 8192 a workgroup is
+// 512 lanes (8 waves), each lane owning two 16-byte vectors (8 bf16 each) of the
+// row in every buffer; it issues its 2*(P+1) loads back to back, so a row keeps
+// (P+1)*16 KiB of HBM reads in flight.
+//
+// Memory policy, measured on MI355X with operands rotated through > 1 GiB:
+//   * partial and residual loads carry the non-temporal bit: the data is used
+//     once, and streaming it past the L2 / last-level cache replacement is worth
+//     ~20 % of bandwidth against default loads;
+//   * residual and output stores are write-through (sc1): the lines leave the L2
+//     while the kernel runs instead of in the write-back at its end (~5 %);
+//   * the weight row is loaded with the default policy and stays cached.
+// Rows are addressed through buffer descriptors whose base is the row and whose
+// extent is one row, so lanes past the end of a short row read zeros and their
+// stores are dropped by the hardware: no tail branches.
+//
+// Rows are walked with stride gridDim.x, so the same kernel serves the
+// one-workgroup-per-row launch (the default: fastest at every size measured) and
+// the capped launch that leaves compute units to a concurrent GEMM.
 //
 // What this replaces in the reference: fused_rs_ln_ag_cta_kernel
 // (csrc/tokenweave_fused_kernels.cu:80-155), fused_rs_ln_cta_kernel and
@@ -103,112 +116,149 @@ __device__ __forceinline__ float inv_rms(float ss, float hidden, float eps) {
 }
 
 // ---------------------------------------------------------------------------
+// Row addressing: one buffer descriptor per (tensor, row).  Offsets inside a row
+// are 32-bit; an access that does not fit inside the row's extent reads zeros /
+// is not written.  Cache-policy bits of the raw buffer intrinsics on gfx950:
+// 1 = sc0, 2 = nt, 16 = sc1.
+// ---------------------------------------------------------------------------
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kLoadStream = 2;    // nt
+constexpr int kLoadCached = 0;
+constexpr int kStoreThrough = 16; // sc1
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_desc(const void* base, size_t row,
+                                                           uint32_t row_bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(static_cast<const char*>(base)) + row * row_bytes, 0, row_bytes, 0x00020000);
+}
+
+template <int AUX>
+__device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t d, uint32_t off) {
+  u32x4_t t = __builtin_amdgcn_raw_buffer_load_b128(d, off, 0, AUX);
+  return make_uint4(t.x, t.y, t.z, t.w);
+}
+
+__device__ __forceinline__ void store16(__amdgpu_buffer_rsrc_t d, uint32_t off, const uint4& v) {
+  u32x4_t t = {v.x, v.y, v.z, v.w};
+  __builtin_amdgcn_raw_buffer_store_b128(t, d, off, 0, kStoreThrough);
+}
+
+// ---------------------------------------------------------------------------
 // Vector kernel, bf16.
 //   NP       number of partial buffers known at compile time, 0 = use np_rt
-//   VPT      16-byte vectors per lane per buffer (row length <= VPT*blockDim*8)
+//   VPT      16-byte vectors per lane per buffer; lane t owns vectors
+//            t, t + blockDim, ... (row length <= VPT * blockDim * 8 elements)
 //   HAS_RES  add the residual and write the rounded sum back to it
 //   COPY     also store the untouched first partial to `copy_out`
 //            (rms_norm_inplace: the copy becomes the residual stream)
 // y may alias any partial: a lane stores y only to vector slots it has already
-// read in every buffer.
+// read in every buffer.  blockDim.x must be a multiple of 64.
 // ---------------------------------------------------------------------------
 template <int NP, int VPT, bool HAS_RES, bool COPY>
 __global__ __launch_bounds__(1024) void row_norm_bf16_kernel(
-    PartialPtrs parts, int np_rt, uint4* y_out, uint4* residual, uint4* copy_out,
-    const uint4* __restrict__ weight, float eps, int num_tokens, int vec_per_row,
-    float hidden) {
+    PartialPtrs parts, int np_rt, void* y_out, void* residual, void* copy_out,
+    const void* __restrict__ weight, float eps, int num_tokens, int vec_per_row, float hidden) {
   __shared__ float slots[2][16];
-  const int tid = threadIdx.x;
   const int nt = blockDim.x;
   const int nwaves = nt >> 6;
   const int np = NP > 0 ? NP : np_rt;
+  const uint32_t row_bytes = (uint32_t)vec_per_row * 16u;
+  uint32_t off[VPT];
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) off[k] = (threadIdx.x + k * nt) * 16u;
 
   uint4 wv[VPT];
+  {
+    const __amdgpu_buffer_rsrc_t dw = row_desc(weight, 0, row_bytes);
 #pragma unroll
-  for (int k = 0; k < VPT; ++k) {
-    const int v = tid + k * nt;
-    wv[k] = v < vec_per_row ? weight[v] : make_uint4(0, 0, 0, 0);
+    for (int k = 0; k < VPT; ++k) wv[k] = load16<kLoadCached>(dw, off[k]);
   }
 
   int phase = 0;
   for (int row = blockIdx.x; row < num_tokens; row += gridDim.x, phase ^= 1) {
-    const size_t base = (size_t)row * vec_per_row;
     float s[VPT][8];
-    float ss = 0.0f;
+    uint4 first[VPT];
+    const __amdgpu_buffer_rsrc_t dr = row_desc(HAS_RES ? residual : y_out, row, row_bytes);
 
-    if (NP > 0) {
-      // Issue every load of the row before the first use.
+    if (NP > 0 && VPT <= 2) {
+      // Issue every load of the row before the first use (at four vectors per
+      // lane that would not fit the register file; those rows accumulate one
+      // partial at a time below).
       uint4 a[VPT][NP > 0 ? NP : 1];
       uint4 rv[VPT];
 #pragma unroll
-      for (int k = 0; k < VPT; ++k) {
-        const int v = tid + k * nt;
-        if (v < vec_per_row) {
+      for (int p = 0; p < NP; ++p) {
+        const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[p], row, row_bytes);
 #pragma unroll
-          for (int p = 0; p < NP; ++p)
-            a[k][p] = static_cast<const uint4*>(parts.p[p])[base + v];
-          if (HAS_RES) rv[k] = residual[base + v];
-        }
+        for (int k = 0; k < VPT; ++k) a[k][p] = load16<kLoadStream>(dp, off[k]);
+      }
+      if (HAS_RES) {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) rv[k] = load16<kLoadStream>(dr, off[k]);
       }
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        const int v = tid + k * nt;
-        if (v < vec_per_row) {
-          unpack8(a[k][0], s[k]);
+        first[k] = a[k][0];
+        unpack8(a[k][0], s[k]);
 #pragma unroll
-          for (int p = 1; p < NP; ++p) add8(a[k][p], s[k]);
-          if (HAS_RES) add8(rv[k], s[k]);
-          if (COPY) copy_out[base + v] = a[k][0];
-        }
+        for (int p = 1; p < NP; ++p) add8(a[k][p], s[k]);
+        if (HAS_RES) add8(rv[k], s[k]);
       }
     } else {
+      {
+        const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[0], row, row_bytes);
 #pragma unroll
-      for (int k = 0; k < VPT; ++k) {
-        const int v = tid + k * nt;
-        if (v < vec_per_row) {
-          uint4 first = static_cast<const uint4*>(parts.p[0])[base + v];
-          unpack8(first, s[k]);
-          for (int p = 1; p < np; ++p)
-            add8(static_cast<const uint4*>(parts.p[p])[base + v], s[k]);
-          if (HAS_RES) add8(residual[base + v], s[k]);
-          if (COPY) copy_out[base + v] = first;
+        for (int k = 0; k < VPT; ++k) {
+          first[k] = load16<kLoadStream>(dp, off[k]);
+          unpack8(first[k], s[k]);
         }
       }
+      for (int p = 1; p < np; ++p) {
+        const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[p], row, row_bytes);
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dp, off[k]), s[k]);
+      }
+      if (HAS_RES) {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dr, off[k]), s[k]);
+      }
+    }
+    if (COPY) {
+      const __amdgpu_buffer_rsrc_t dc = row_desc(copy_out, row, row_bytes);
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) store16(dc, off[k], first[k]);
     }
 
     // Sum of squares of the unrounded fp32 sum; round the residual once.
+    // (Lanes past the row's end hold zeros and add nothing.)
+    float ss = 0.0f;
     uint4 rnew[VPT];
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
-      const int v = tid + k * nt;
-      if (v < vec_per_row) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) ss += s[k][e] * s[k][e];
-        rnew[k].x = pack_bf16(s[k][0], s[k][1]);
-        rnew[k].y = pack_bf16(s[k][2], s[k][3]);
-        rnew[k].z = pack_bf16(s[k][4], s[k][5]);
-        rnew[k].w = pack_bf16(s[k][6], s[k][7]);
-        if (HAS_RES) residual[base + v] = rnew[k];
-      }
+      for (int e = 0; e < 8; ++e) ss += s[k][e] * s[k][e];
+      rnew[k].x = pack_bf16(s[k][0], s[k][1]);
+      rnew[k].y = pack_bf16(s[k][2], s[k][3]);
+      rnew[k].z = pack_bf16(s[k][4], s[k][5]);
+      rnew[k].w = pack_bf16(s[k][6], s[k][7]);
+      if (HAS_RES) store16(dr, off[k], rnew[k]);
     }
 
     const float total = block_sum(ss, slots[phase], nwaves);
     const float inv = inv_rms(total, hidden, eps);
 
+    const __amdgpu_buffer_rsrc_t dy = row_desc(y_out, row, row_bytes);
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
-      const int v = tid + k * nt;
-      if (v < vec_per_row) {
-        float r[8], w[8];
-        unpack8(rnew[k], r);
-        unpack8(wv[k], w);
-        uint4 o;
-        o.x = pack_bf16(r[0] * inv * w[0], r[1] * inv * w[1]);
-        o.y = pack_bf16(r[2] * inv * w[2], r[3] * inv * w[3]);
-        o.z = pack_bf16(r[4] * inv * w[4], r[5] * inv * w[5]);
-        o.w = pack_bf16(r[6] * inv * w[6], r[7] * inv * w[7]);
-        y_out[base + v] = o;
-      }
+      float r[8], w[8];
+      unpack8(rnew[k], r);
+      unpack8(wv[k], w);
+      uint4 o;
+      o.x = pack_bf16(r[0] * inv * w[0], r[1] * inv * w[1]);
+      o.y = pack_bf16(r[2] * inv * w[2], r[3] * inv * w[3]);
+      o.z = pack_bf16(r[4] * inv * w[4], r[5] * inv * w[5]);
+      o.w = pack_bf16(r[6] * inv * w[6], r[7] * inv * w[7]);
+      store16(dy, off[k], o);
     }
   }
 }
@@ -275,12 +325,26 @@ __global__ __launch_bounds__(1024) void row_norm_elem_kernel(
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 static int default_grid(int64_t num_tokens) {
-  // One workgroup per row until the rows outnumber what the device keeps
-  // resident (two 1024-lane workgroups per compute unit); beyond that the
-  // resident workgroups walk the rows.
-  const int cus = device_compute_units();
-  const int64_t resident = (int64_t)(cus > 0 ? cus : 256) * 2;
-  return (int)(num_tokens < resident ? num_tokens : resident);
+  // One workgroup per row.  Measured against grids capped at 1x .. 8x the
+  // compute-unit count, the uncapped launch is as fast or faster at every size
+  // from 1 to 8192 rows: the hardware dispatcher refills a compute unit as soon as
+  // a row retires, which beats a fixed row-to-workgroup assignment.
+  return (int)(num_tokens < INT32_MAX ? num_tokens : INT32_MAX);
+}
+
+// Lanes and vectors per lane for a row of V 16-byte vectors.  The choice depends
+// on V only, never on the token count or the grid, so a row's result does not
+// depend on the launch.  V <= 256: one vector per lane; up to 2048: two (512
+// lanes at hidden size 8192, the best shape from 256 to 3001 rows); up to 4096:
+// four.  Longer rows take the element-wise kernel.
+static bool vec_shape(int V, int* vpt, int* nt) {
+  int v = V <= 256 ? 1 : V <= 2048 ? 2 : V <= 4096 ? 4 : 0;
+  if (v == 0) return false;
+  int lanes = (V + v - 1) / v;
+  lanes = ((lanes + 63) / 64) * 64;
+  *vpt = v;
+  *nt = lanes;
+  return true;
 }
 
 template <int NP, bool HAS_RES, bool COPY>
@@ -288,18 +352,15 @@ static int launch_vec_vpt(const PartialPtrs& parts, int np, void* y, void* resid
                           void* copy_out, const void* weight, int64_t T, int64_t H,
                           float eps, int grid, hipStream_t stream) {
   const int V = (int)(H / 8);
-  int nt = V < 1024 ? ((V + 63) / 64) * 64 : 1024;
-  const int vpt = (V + nt - 1) / nt;
+  int vpt = 0, nt = 0;
+  if (!vec_shape(V, &vpt, &nt)) return 1;  // caller falls back to the element-wise kernel
   dim3 g(grid), b(nt);
-#define TW_LAUNCH(VPT)                                                              \
-  hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, HAS_RES, COPY>), g, b, 0, stream, \
-                     parts, np, static_cast<uint4*>(y), static_cast<uint4*>(residual), \
-                     static_cast<uint4*>(copy_out), static_cast<const uint4*>(weight), \
-                     eps, (int)T, V, (float)H)
+#define TW_LAUNCH(VPT)                                                                  \
+  hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, HAS_RES, COPY>), g, b, 0, stream,   \
+                     parts, np, y, residual, copy_out, weight, eps, (int)T, V, (float)H)
   if (vpt == 1) TW_LAUNCH(1);
   else if (vpt == 2) TW_LAUNCH(2);
-  else if (vpt <= 4) TW_LAUNCH(4);
-  else return 1;  // caller falls back to the element-wise kernel
+  else TW_LAUNCH(4);
 #undef TW_LAUNCH
   return 0;
 }

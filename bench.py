@@ -6,9 +6,12 @@
 A step is one call of the fused op (one kernel launch) on one batch of synthetic
 input that is already resident in HBM.  The default workload is the headline
 configuration: one rank's shard of a Llama-70B TP=8 layer, P=8 partials of
-[256, 8192] bf16 (a T=2048 batch).  Consecutive steps use different input sets
-(rotation over more than 1 GiB) so that no step finds its operands in the 256 MB
-last-level cache.  Prints ONE JSON line on stdout; progress goes to stderr.
+[256, 8192] bf16 (a T=2048 batch).  Consecutive steps use different input sets,
+cycling through 4 GiB of operands before any reuse.  The footprint is that large
+on purpose: the kernel's streaming loads do not allocate in the 256 MB last-level
+cache, so with a ~1 GiB rotation the lines WRITTEN by earlier steps (residual and
+output) survive there until their set comes round again and inflate the figure by
+up to 15 %.  Prints ONE JSON line on stdout; progress goes to stderr.
 
 Fields beyond the usual ones:
   roofline      HBM roofline of the norm kernel: algorithmic bytes per launch
@@ -34,7 +37,13 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-ROTATION_BYTES = (1 << 30) + (1 << 28) # > 1 GiB of distinct operands before any reuse
+ROTATION_BYTES = 4 << 30      # distinct operand bytes cycled through before any reuse
+
+# HBM bytes per launch read from the hardware counters (rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE, each scaled by the same counter's reading for the library's plain copy
+# kernel of known size); the runs are summarised in
+# profiles/row_norm_bf16_c2_T256_pmc_traffic.md.  Workloads without a counter run: None.
+MEASURED_TRAFFIC_BYTES = {"c2_llama70b_tp8_shard@T256": 46373129}
 
 
 def log(*a):
@@ -50,6 +59,9 @@ def parse_args():
     ap.add_argument("--max-ctas", type=int, default=0, help="grid cap (0 = library default)")
     ap.add_argument("--sweep", action="store_true", help="also time every configuration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="after the timed region, run the library's plain copy kernel on "
+                         "buffers of known size (reference traffic for rocprofv3 --pmc runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline")
     return ap.parse_args()
 
@@ -89,7 +101,7 @@ def time_norm(cfg, steps, warmup, max_ctas, device):
     two synchronisation points, and the mean launch duration from the HIP events that
     bracket the same `steps` back-to-back launches."""
     import torch
-    nsets = max(2, min(64, -(-ROTATION_BYTES // cfg.bytes)))
+    nsets = max(2, min(256, -(-ROTATION_BYTES // cfg.bytes)))
     free, _ = torch.cuda.mem_get_info()
     set_bytes = (cfg.P + 1) * cfg.T * cfg.H * 2 + cfg.H * 2
     nsets = max(2, min(nsets, int(free * 0.6) // (set_bytes * 3)))  # fp32 staging while generating
@@ -114,6 +126,44 @@ def time_norm(cfg, steps, warmup, max_ctas, device):
     del runner
     torch.cuda.empty_cache()
     return res
+
+
+CALIBRATION_COPY_BYTES = 256 << 20
+
+
+def calibration_copies(device, n=8):
+    """n launches of tw_copy_bytes, each reading and writing CALIBRATION_COPY_BYTES of
+    memory that was not touched recently (4 source/destination pairs = 2 GiB)."""
+    import torch
+    from tokenweave_amd import _custom_ops as ops
+    pairs = [(torch.ones(CALIBRATION_COPY_BYTES // 2, dtype=torch.bfloat16, device=device),
+              torch.empty(CALIBRATION_COPY_BYTES // 2, dtype=torch.bfloat16, device=device))
+             for _ in range(4)]
+    torch.cuda.synchronize()
+    for i in range(n):
+        src, dst = pairs[i % 4]
+        ops.copy_bytes(dst, src)
+    torch.cuda.synchronize()
+
+
+def time_norm_warm(cfg, steps, max_ctas, device):
+    """Same call on ONE input set, so that after the first step the operands sit in
+    the last-level cache (what a caller sees when the partials were just written)."""
+    import torch
+    runner = NormRunner(cfg, 1, max_ctas, device)
+    stream = torch.cuda.current_stream()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    for i in range(10):
+        runner.step(0, sp)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for i in range(steps):
+        runner.step(0, sp)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    del runner
+    torch.cuda.empty_cache()
+    return e0.elapsed_time(e1) * 1e3 / steps
 
 
 def cpu_baseline(cfg, budget_s):
@@ -225,21 +275,28 @@ def main():
         "pct_hbm_peak": round(100.0 * res["gbps"] / HBM_PEAK_GBPS, 2),
         "us_per_call": round(res["ms_per_step"] * 1e3, 3),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "row_norm_bf16_kernel<8,2,true,false>",
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name) if args.max_ctas == 0 else None,
+                     "kernel": "row_norm_bf16_kernel<8,4,256,true,false>",
                      "kernel_us_mean": round(kernel_us, 3)},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
         log(f"[bench] cpu_baseline {out['cpu_baseline']}")
+    if args.calibration_copy:
+        calibration_copies(device)
     if args.sweep:
         sweep = {}
+        cfgs = dict(cfgs)
+        cfgs["c2_unsharded@T2048"] = wl.C2.with_tokens(2048, "c2_unsharded@T2048")
         for name, c in cfgs.items():
-            steps = max(20, min(args.steps, int(2e9 // c.bytes)))
+            steps = max(50, min(2000, int(0.02 * 5e12 / c.bytes)))  # ~20 ms of kernel time
             r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device)
+            warm_us = time_norm_warm(c, steps, args.max_ctas, device) if c.bytes < (200 << 20) else None
             sweep[name] = {"P": c.P, "T": c.T, "H": c.H, "bytes": c.bytes,
                            "us_per_call": round(r["ms_per_step"] * 1e3, 3),
                            "kernel_us": round(r["kernel_us_mean"], 3),
+                           "kernel_us_cache_resident": None if warm_us is None else round(warm_us, 3),
                            "gbps": round(c.bytes / r["kernel_us_mean"] / 1e3, 1),
                            "pct_hbm_peak": round(c.bytes / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
             log(f"[sweep] {name}: {sweep[name]}")

@@ -143,6 +143,13 @@ TW_API int tw_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M,
                     int64_t N, int64_t K, int64_t ldc, int max_cus,
                     void* stream);
 
+/* dst[0, nbytes) <- src[0, nbytes) with a plain grid-stride copy kernel (default
+ * cache policy, 16 bytes per lane).  nbytes % 16 == 0, 16-byte aligned pointers,
+ * non-overlapping ranges.  A measurement utility with no counterpart in the
+ * reference: its traffic is known exactly, so hardware memory counters read for
+ * the norm kernels can be scaled against it. */
+TW_API int tw_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -284,6 +284,16 @@ def gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
                                               ldc, _cap(max_cus), _stream_ptr(a)))
 
 
+def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """dst <- src through the library's plain copy kernel (counter calibration)."""
+    _require(dst.is_cuda and src.is_cuda and dst.device == src.device, "copy needs two tensors on one GPU")
+    _require(dst.is_contiguous() and src.is_contiguous(), "copy needs contiguous tensors")
+    nbytes = src.numel() * src.element_size()
+    _require(nbytes == dst.numel() * dst.element_size(), "copy needs equally sized tensors")
+    with _on_device(dst):
+        _lib.check(_lib.lib().tw_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, _stream_ptr(dst)))
+
+
 def num_compute_units(device=None) -> int:
     dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
     with torch.cuda.device(dev):

@@ -39,6 +39,7 @@ PROTOTYPES = {
     "tw_fused_rs_ln_cta": [_vp, _vp, _vp, _u64, _i64, _ci, _ci, _ci, _f32, _i64, _i64, _vp],
     "tw_fused_rs_ln_ag_cta": [_vp, _vp, _vp, _u64, _i64, _ci, _ci, _ci, _f32, _i64, _i64, _vp],
     "tw_gemm_bf16_nt": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp],
+    "tw_copy_bytes": [_vp, _vp, _i64, _vp],
 }
 
 _lib = None

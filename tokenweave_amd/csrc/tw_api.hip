@@ -137,6 +137,10 @@ int tw_fused_rs_ln_ag_cta(void* input, void* residual, const void* weight, uint6
                           stream);
 }
 
+int tw_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
+  return tw::run_copy16(dst, src, nbytes, stream);
+}
+
 int tw_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t N, int64_t K,
                     int64_t ldc, int max_cus, void* stream) {
   return tw::run_gemm_bf16_nt(out, a, b, M, N, K, ldc, max_cus, stream);

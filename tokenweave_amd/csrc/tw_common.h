@@ -20,6 +20,8 @@ int run_row_norm(const char* what, const void* const* partials, int np, void* y,
                  int64_t H, float eps, int dtype, int max_ctas, bool require_vec,
                  void* stream);
 
+int run_copy16(void* dst, const void* src, int64_t nbytes, void* stream);
+
 int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t N,
                      int64_t K, int64_t ldc, int max_cus, void* stream);
 

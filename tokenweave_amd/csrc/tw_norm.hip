@@ -2,17 +2,18 @@
 //
 // One workgroup owns one token row at a time and keeps the whole row in
 // registers between the sum-of-squares reduction and the normalised store:
-// every byte is read once and written once.  At hidden size 8192 a workgroup is
-// 512 lanes (8 waves), each lane owning two 16-byte vectors (8 bf16 each) of the
-// row in every buffer; it issues its 2*(P+1) loads back to back, so a row keeps
-// (P+1)*16 KiB of HBM reads in flight.
+// every byte is read once and written once.  At hidden size 8192 and 64 rows or
+// more a workgroup is 256 lanes (4 waves), each lane owning four 16-byte vectors
+// (8 bf16 each) of the row in every buffer; it issues its 4*(P+1) loads back to
+// back, so a row keeps (P+1)*16 KiB of HBM reads in flight.  With fewer rows a
+// row is spread over 1024 lanes, one vector each.
 //
 // Memory policy, measured on MI355X with operands rotated through > 1 GiB:
 //   * partial and residual loads carry the non-temporal bit: the data is used
 //     once, and streaming it past the L2 / last-level cache replacement is worth
 //     ~20 % of bandwidth against default loads;
-//   * residual and output stores are write-through (sc1): the lines leave the L2
-//     while the kernel runs instead of in the write-back at its end (~5 %);
+//   * residual and output stores carry it too: the lines leave the L2 while the
+//     kernel runs instead of in the write-back at its end (~10 % at 2048 rows);
 //   * the weight row is loaded with the default policy and stays cached.
 // Rows are addressed through buffer descriptors whose base is the row and whose
 // extent is one row, so lanes past the end of a short row read zeros and their
@@ -71,15 +72,23 @@ __device__ __forceinline__ void add8(const uint4& v, float (&f)[8]) {
 }
 
 // ---------------------------------------------------------------------------
-// Sum over the workgroup, result in every lane.  Fixed order, so a row's sum
-// depends only on the row's data and on blockDim.x.
-//   lanes:  xor-1, xor-2 (quad permutes), half-row mirror, row mirror on DPP —
-//           every lane of a 16-lane row then holds that row's sum;
-//   rows:   ((row0 + row1) + row2) + row3 through v_readlane;
-//   waves:  one LDS slot per wave, one barrier, every lane adds the slots in
-//           wave order (broadcast reads).
-// `slots` must hold 16 floats and must not be reused before the next barrier
-// (callers alternate between two slot arrays).
+// Sums with a fixed association order.
+//
+// wave_sum: 64 lanes -> the same total in every lane.  xor-1, xor-2 (quad
+//   permutes), half-row mirror, row mirror on DPP leave every lane of a 16-lane
+//   row with that row's sum; the four row sums are added as ((r0+r1)+r2)+r3
+//   through v_readlane.
+// block_sum (element-wise kernel): wave sums through one LDS slot per wave, one
+//   barrier, every lane adds the slots in wave order.
+// row_sum_chunks (vector kernel): the row is cut into chunks of 64 consecutive
+//   16-byte vectors; chunk c is reduced with wave_sum by whichever wave owns it,
+//   and the (at most 64) chunk sums, one per lane, are reduced with wave_sum again.  Lane t of a workgroup of
+//   nt lanes owns vectors t, t + nt, ... (nt a multiple of 64), so the chunk of
+//   its k-th vector is k * nt/64 + wave.  The result therefore depends only on
+//   the row's data — not on the workgroup size or the vectors per lane — which
+//   lets the launcher pick the workgroup shape per token count.
+// LDS slots must not be reused before the next barrier (callers alternate
+// between two slot arrays).
 // ---------------------------------------------------------------------------
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
@@ -109,6 +118,25 @@ __device__ __forceinline__ float block_sum(float v, float* slots, int nwaves) {
   return total;
 }
 
+constexpr int kMaxChunks = 64;  // 4096 vectors = hidden size 32768
+
+template <int VPT>
+__device__ __forceinline__ float row_sum_chunks(const float (&per_vec)[VPT], float* slots,
+                                                int nwaves, int nchunks) {
+  const int wave = threadIdx.x >> 6;
+  float c[VPT];
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) c[k] = wave_sum(per_vec[k]);
+  if (VPT == 1 && nwaves == 1) return c[0];
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) slots[k * nwaves + wave] = c[k];
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63;
+  return wave_sum(lane < nchunks ? slots[lane] : 0.0f);
+}
+
 __device__ __forceinline__ float inv_rms(float ss, float hidden, float eps) {
   // Same expression as csrc/cpu/layernorm.cpp:72-73; hipcc keeps fp32 division
   // and sqrt correctly rounded.
@@ -124,7 +152,7 @@ __device__ __forceinline__ float inv_rms(float ss, float hidden, float eps) {
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int kLoadStream = 2;    // nt
 constexpr int kLoadCached = 0;
-constexpr int kStoreThrough = 16; // sc1
+constexpr int kStoreStream = 2;  // nt
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t row_desc(const void* base, size_t row,
                                                            uint32_t row_bytes) {
@@ -140,7 +168,7 @@ __device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t d, uint32_t off) 
 
 __device__ __forceinline__ void store16(__amdgpu_buffer_rsrc_t d, uint32_t off, const uint4& v) {
   u32x4_t t = {v.x, v.y, v.z, v.w};
-  __builtin_amdgcn_raw_buffer_store_b128(t, d, off, 0, kStoreThrough);
+  __builtin_amdgcn_raw_buffer_store_b128(t, d, off, 0, kStoreStream);
 }
 
 // ---------------------------------------------------------------------------
@@ -154,25 +182,21 @@ __device__ __forceinline__ void store16(__amdgpu_buffer_rsrc_t d, uint32_t off, 
 // y may alias any partial: a lane stores y only to vector slots it has already
 // read in every buffer.  blockDim.x must be a multiple of 64.
 // ---------------------------------------------------------------------------
-template <int NP, int VPT, bool HAS_RES, bool COPY>
-__global__ __launch_bounds__(1024) void row_norm_bf16_kernel(
+template <int NP, int VPT, int MAXNT, bool HAS_RES, bool COPY>
+__global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
     PartialPtrs parts, int np_rt, void* y_out, void* residual, void* copy_out,
     const void* __restrict__ weight, float eps, int num_tokens, int vec_per_row, float hidden) {
-  __shared__ float slots[2][16];
+  __shared__ float slots[2][kMaxChunks];
   const int nt = blockDim.x;
   const int nwaves = nt >> 6;
+  const int nchunks = (vec_per_row + 63) >> 6;  // <= VPT * nwaves
   const int np = NP > 0 ? NP : np_rt;
   const uint32_t row_bytes = (uint32_t)vec_per_row * 16u;
   uint32_t off[VPT];
 #pragma unroll
   for (int k = 0; k < VPT; ++k) off[k] = (threadIdx.x + k * nt) * 16u;
 
-  uint4 wv[VPT];
-  {
-    const __amdgpu_buffer_rsrc_t dw = row_desc(weight, 0, row_bytes);
-#pragma unroll
-    for (int k = 0; k < VPT; ++k) wv[k] = load16<kLoadCached>(dw, off[k]);
-  }
+  const __amdgpu_buffer_rsrc_t dw = row_desc(weight, 0, row_bytes);
 
   int phase = 0;
   for (int row = blockIdx.x; row < num_tokens; row += gridDim.x, phase ^= 1) {
@@ -180,10 +204,10 @@ __global__ __launch_bounds__(1024) void row_norm_bf16_kernel(
     uint4 first[VPT];
     const __amdgpu_buffer_rsrc_t dr = row_desc(HAS_RES ? residual : y_out, row, row_bytes);
 
-    if (NP > 0 && VPT <= 2) {
-      // Issue every load of the row before the first use (at four vectors per
-      // lane that would not fit the register file; those rows accumulate one
-      // partial at a time below).
+    if (NP > 0 && (VPT <= 2 || MAXNT <= 256)) {
+      // Issue every load of the row before the first use.  (Four vectors per lane
+      // in a workgroup of more than 256 lanes would not fit the register file;
+      // those rows accumulate one partial at a time below.)
       uint4 a[VPT][NP > 0 ? NP : 1];
       uint4 rv[VPT];
 #pragma unroll
@@ -223,20 +247,28 @@ __global__ __launch_bounds__(1024) void row_norm_bf16_kernel(
         for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dr, off[k]), s[k]);
       }
     }
+    // The weight row is fetched per token row, behind the row's own loads: it is
+    // an L2 hit after the first workgroups, and fetching it up front would put
+    // its (cold) latency ahead of the first partial load.
+    uint4 wv[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) wv[k] = load16<kLoadCached>(dw, off[k]);
+
     if (COPY) {
       const __amdgpu_buffer_rsrc_t dc = row_desc(copy_out, row, row_bytes);
 #pragma unroll
       for (int k = 0; k < VPT; ++k) store16(dc, off[k], first[k]);
     }
 
-    // Sum of squares of the unrounded fp32 sum; round the residual once.
-    // (Lanes past the row's end hold zeros and add nothing.)
-    float ss = 0.0f;
+    // Sum of squares of the unrounded fp32 sum, one running sum per vector; round
+    // the residual once.  (Lanes past the row's end hold zeros and add nothing.)
+    float ss[VPT];
     uint4 rnew[VPT];
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
+      ss[k] = 0.0f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ss += s[k][e] * s[k][e];
+      for (int e = 0; e < 8; ++e) ss[k] += s[k][e] * s[k][e];
       rnew[k].x = pack_bf16(s[k][0], s[k][1]);
       rnew[k].y = pack_bf16(s[k][2], s[k][3]);
       rnew[k].z = pack_bf16(s[k][4], s[k][5]);
@@ -244,7 +276,7 @@ __global__ __launch_bounds__(1024) void row_norm_bf16_kernel(
       if (HAS_RES) store16(dr, off[k], rnew[k]);
     }
 
-    const float total = block_sum(ss, slots[phase], nwaves);
+    const float total = row_sum_chunks<VPT>(ss, slots[phase], nwaves, nchunks);
     const float inv = inv_rms(total, hidden, eps);
 
     const __amdgpu_buffer_rsrc_t dy = row_desc(y_out, row, row_bytes);
@@ -332,18 +364,30 @@ static int default_grid(int64_t num_tokens) {
   return (int)(num_tokens < INT32_MAX ? num_tokens : INT32_MAX);
 }
 
-// Lanes and vectors per lane for a row of V 16-byte vectors.  The choice depends
-// on V only, never on the token count or the grid, so a row's result does not
-// depend on the launch.  V <= 256: one vector per lane; up to 2048: two (512
-// lanes at hidden size 8192, the best shape from 256 to 3001 rows); up to 4096:
-// four.  Longer rows take the element-wise kernel.
-static bool vec_shape(int V, int* vpt, int* nt) {
-  int v = V <= 256 ? 1 : V <= 2048 ? 2 : V <= 4096 ? 4 : 0;
-  if (v == 0) return false;
-  int lanes = (V + v - 1) / v;
-  lanes = ((lanes + 63) / 64) * 64;
-  *vpt = v;
-  *nt = lanes;
+// Workgroup shape for rows of V 16-byte vectors and T rows.  Results do not
+// depend on the shape (row_sum_chunks), so it is chosen for speed alone:
+//   * few rows (T < 64): as many lanes per row as the row has vectors (up to
+//     1024), one or two vectors each — the shortest path from launch to the last
+//     store when the call is latency bound;
+//   * many rows: four vectors per lane in workgroups of at most 256 lanes, every
+//     load of the row in flight at once (the fastest shape measured from 256 to
+//     8192 rows at hidden sizes 6144 and 8192);
+//   * rows longer than 1024 vectors: two vectors per lane up to 2048 vectors, four
+//     up to 4096 (one partial at a time).  Longer rows take the element-wise kernel.
+struct VecShape { int vpt, nt, maxnt; };
+
+static bool vec_shape(int V, int64_t T, VecShape* sh) {
+  int vpt, maxnt = 1024;
+  if (V <= 1024) {
+    if (T < 64 || V < 256) vpt = 1;
+    else { vpt = 4; maxnt = 256; }
+  } else if (V <= 2048) vpt = 2;
+  else if (V <= 4096) vpt = 4;
+  else return false;
+  int lanes = (V + vpt - 1) / vpt;
+  sh->vpt = vpt;
+  sh->nt = ((lanes + 63) / 64) * 64;
+  sh->maxnt = maxnt;
   return true;
 }
 
@@ -352,15 +396,16 @@ static int launch_vec_vpt(const PartialPtrs& parts, int np, void* y, void* resid
                           void* copy_out, const void* weight, int64_t T, int64_t H,
                           float eps, int grid, hipStream_t stream) {
   const int V = (int)(H / 8);
-  int vpt = 0, nt = 0;
-  if (!vec_shape(V, &vpt, &nt)) return 1;  // caller falls back to the element-wise kernel
-  dim3 g(grid), b(nt);
-#define TW_LAUNCH(VPT)                                                                  \
-  hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, HAS_RES, COPY>), g, b, 0, stream,   \
+  VecShape sh;
+  if (!vec_shape(V, T, &sh)) return 1;  // caller falls back to the element-wise kernel
+  dim3 g(grid), b(sh.nt);
+#define TW_LAUNCH(VPT, MAXNT)                                                                  \
+  hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, MAXNT, HAS_RES, COPY>), g, b, 0, stream,   \
                      parts, np, y, residual, copy_out, weight, eps, (int)T, V, (float)H)
-  if (vpt == 1) TW_LAUNCH(1);
-  else if (vpt == 2) TW_LAUNCH(2);
-  else TW_LAUNCH(4);
+  if (sh.vpt == 1) TW_LAUNCH(1, 1024);
+  else if (sh.vpt == 2) TW_LAUNCH(2, 1024);
+  else if (sh.maxnt == 256) TW_LAUNCH(4, 256);
+  else TW_LAUNCH(4, 1024);
 #undef TW_LAUNCH
   return 0;
 }
@@ -461,6 +506,37 @@ int run_row_norm(const char* what, const void* const* partials, int np, void* y,
       break;
   }
   return finish_launch(what);
+}
+
+// ---------------------------------------------------------------------------
+// Plain copy with default cache policy: the known-size traffic against which
+// hardware memory counters are scaled.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void copy16_kernel(uint4* __restrict__ dst,
+                                                     const uint4* __restrict__ src, size_t n) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
+int run_copy16(void* dst, const void* src, int64_t nbytes, void* stream) {
+  if (nbytes < 0 || nbytes % 16 != 0)
+    return set_error(TW_ERR_INVALID_ARGUMENT, "copy: byte count %lld is not a non-negative multiple of 16",
+                     (long long)nbytes);
+  if (nbytes == 0) return TW_OK;
+  if (!dst || !src) return set_error(TW_ERR_INVALID_ARGUMENT, "copy: null pointer argument");
+  if ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u)
+    return set_error(TW_ERR_ALIGNMENT, "copy: pointers must be 16-byte aligned");
+  const size_t n = (size_t)nbytes / 16;
+  const int cus = device_compute_units();
+  size_t blocks = (n + 255) / 256;
+  const size_t cap = (size_t)(cus > 0 ? cus : 256) * 16;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<uint4*>(dst), static_cast<const uint4*>(src), n);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return set_error(TW_ERR_LAUNCH, "copy: kernel launch failed: %s", hipGetErrorString(e));
+  return TW_OK;
 }
 
 }  // namespace tw

@@ -30,22 +30,30 @@ class PartialsBuffer:
     """
 
     def __init__(self, world_size: int, max_tokens: int, hidden_size: int, rank: int = 0,
-                 device: Any = "cuda", dtype: torch.dtype = torch.bfloat16) -> None:
+                 device: Any = "cuda", dtype: torch.dtype = torch.bfloat16,
+                 slot_pad_bytes: int = 0) -> None:
         assert 0 <= rank < world_size, f"Invalid rank {rank}, must be in [0, {world_size - 1}]"
         if dtype != torch.bfloat16:
             raise NotImplementedError("staging buffers are bf16, like the reference's")
         if hidden_size % 8 != 0:
             raise RuntimeError(ops.ALIGNMENT_MESSAGE)
+        if slot_pad_bytes < 0 or slot_pad_bytes % 16 != 0:
+            raise ValueError("slot_pad_bytes must be a non-negative multiple of 16")
         self.world_size = world_size
         self.rank = rank
         self.max_tokens = max_tokens
         self.hidden_size = hidden_size
-        self.storage = torch.empty(world_size, max_tokens, hidden_size, dtype=dtype, device=device)
-        self.peer_stride_bytes = max_tokens * hidden_size * self.storage.element_size()
-        self.multicast_ptr = self.storage.data_ptr()
+        # slot_pad_bytes spaces the slots apart, for callers that want the P streams of
+        # one row to fall on different memory channels
+        slot_elems = max_tokens * hidden_size + slot_pad_bytes // 2
+        self._backing = torch.empty(world_size * slot_elems, dtype=dtype, device=device)
+        self.storage = self._backing.as_strided((world_size, max_tokens, hidden_size),
+                                                (slot_elems, hidden_size, 1))
+        self.peer_stride_bytes = slot_elems * 2
+        self.multicast_ptr = self._backing.data_ptr()
         self.signal_pad_ptrs_dev = 0
         ops.register_partials_region(self.multicast_ptr, self.peer_stride_bytes, world_size,
-                                     self.storage)
+                                     self._backing)
 
     def slot(self, p: int) -> torch.Tensor:
         """Rank p's staging buffer, [max_tokens, hidden_size]."""

@@ -104,10 +104,10 @@ def test_weave_step_equals_serial_execution():
     torch.cuda.synchronize()
     buf2, res2 = setup()
     side = torch.cuda.Stream()
-    for _ in range(3):  # the step is idempotent on split A and we reset split B each time
+    for gemm_first in (True, False, True):  # the step is idempotent on split A; split B is reset each time
         buf2.storage[:, Ta:] = inp.staging
         res2[Ta:] = inp.residual
-        tw.weave_norm_gemm(lambda: gemm(buf2), lambda: norm(buf2, res2), side)
+        tw.weave_norm_gemm(lambda: gemm(buf2), lambda: norm(buf2, res2), side, gemm_first=gemm_first)
         torch.cuda.synchronize()
         assert torch.equal(buf1.storage, buf2.storage) and torch.equal(res1, res2)
     check(buf2.local[:Ta], g.a, g.b, "weave gemm split")

@@ -280,6 +280,30 @@ def test_runs_on_the_current_torch_stream(oracle):
     assert np.array_equal(to_bits(out), y0) and np.array_equal(to_bits(res), r0)
 
 
+def test_op_is_capturable_in_a_hip_graph_and_replays_exactly():
+    """The entry points only enqueue (no allocation, no host sync), so a caller may
+    capture them.  Every replay is checked against the eager result, with eager work
+    and synchronisations between replays."""
+    inp = wl.make_norm_inputs(wl.C2.with_tokens(96), DEV)
+    y0, r0, _ = run_hip(inp)
+    parts = [p.clone() for p in inp.partials]
+    res, out = inp.residual.clone(), torch.empty_like(inp.residual)
+    cap = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=cap):
+        ops.reduce_add_rms_norm(parts, out, res, inp.weight, inp.cfg.eps)
+    for i in range(4):
+        res.copy_(inp.residual)      # eager work between replays: the op mutates the residual
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(to_bits(out), y0) and np.array_equal(to_bits(res), r0), f"replay {i}"
+        y_e, r_e, _ = run_hip(inp)   # eager call of the same op between replays
+        assert np.array_equal(y_e, y0) and np.array_equal(r_e, r0)
+
+
 def test_argument_errors_on_device_tensors():
     H = 64
     x = torch.zeros(8, H, dtype=torch.bfloat16, device=DEV)

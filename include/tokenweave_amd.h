@@ -143,6 +143,37 @@ TW_API int tw_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M,
                     int64_t N, int64_t K, int64_t ldc, int max_cus,
                     void* stream);
 
+/* Norm with static-scale fp8 output.  out is [num_tokens, hidden_size] of OCP
+ * float8 e4m3fn (1 byte per element): out = fp8_rne(clamp(y / *scale, +-448)),
+ * where y is the bf16 (or `dtype`) result the unquantised op would store, and
+ * `scale` points to ONE fp32 value in device memory.  input is not modified.
+ * Replaces ::rms_norm_static_fp8_quant (csrc/layernorm_quant_kernels.cu:165-190,
+ * schema at csrc/torch_bindings.cpp:199-205). */
+TW_API int tw_rms_norm_static_fp8_quant(void* out, const void* input, const void* weight,
+                                        const float* scale, int64_t num_tokens,
+                                        int64_t hidden_size, float epsilon, int dtype,
+                                        void* stream);
+
+/* residual <- input + residual ; out <- fp8 quantisation (as above) of
+ * RMSNorm(residual) * weight.  input is not modified.
+ * Replaces ::fused_add_rms_norm_static_fp8_quant
+ * (csrc/layernorm_quant_kernels.cu:203-245, schema at
+ * csrc/torch_bindings.cpp:207-213). */
+TW_API int tw_fused_add_rms_norm_static_fp8_quant(void* out, const void* input, void* residual,
+                                                  const void* weight, const float* scale,
+                                                  int64_t num_tokens, int64_t hidden_size,
+                                                  float epsilon, int dtype, void* stream);
+
+/* tw_reduce_add_rms_norm with the fp8 output above: the fused P-partial op
+ * feeding an fp8 GEMM.  bf16 in; 16-byte alignment and hidden_size % 16 == 0
+ * required.  No counterpart in the reference (its TokenWeave kernels emit bf16);
+ * it composes the two reference ops it is named after. */
+TW_API int tw_reduce_add_rms_norm_static_fp8_quant(const void* const* partials, int num_partials,
+                                                   void* out, void* residual, const void* weight,
+                                                   const float* scale, int64_t num_tokens,
+                                                   int64_t hidden_size, int max_ctas,
+                                                   float epsilon, void* stream);
+
 /* dst[0, nbytes) <- src[0, nbytes) with a plain grid-stride copy kernel (default
  * cache policy, 16 bytes per lane).  nbytes % 16 == 0, 16-byte aligned pointers,
  * non-overlapping ranges.  A measurement utility with no counterpart in the

@@ -16,11 +16,14 @@
  *   csrc/custom_all_reduce.cuh:286-294  P-way sum: fp32, fixed order p = 0..P-1,
  *                                  one down-cast at the end
  *   csrc/tokenweave_fused_kernels.cu:37-72  rms_norm_inplace (copy + normalise)
+ *   csrc/quantization/fp8/common.cuh:38-56  static-scale fp8 conversion (the
+ *                                  reference has no CPU twin of the norm+quant ops)
  *
  * Pinned by (tests/test_oracle_*.py): bit equality with the reference's own
  * layernorm.cpp compiled from its sources (oracle/_ref, truncating build) on the
  * reference's test grid; closed forms (constant / one-hot / zero rows); an
- * independent numpy fp32 restatement of RMSNorm.forward_native; float64 witness.
+ * independent numpy fp32 restatement of RMSNorm.forward_native; float64 witness;
+ * the fp8 conversion against torch's own CPU cast over every bf16 bit pattern.
  *
  * Every function is built with -ffp-contract=off: the reference's vector code is
  * separate multiplies and adds (no FMA in its AVX2 build).
@@ -128,6 +131,46 @@ int tw_oracle_rms_norm_inplace(uint16_t* out, uint16_t* x, const uint16_t* w,
     memcpy(out + i * H, x + i * H, (size_t)H * 2);
     const uint16_t* parts[1] = {x};
     row_reduce_add_norm(parts, 0, i * H, 0, x + i * H, w, eps, (int)H, mode);
+  }
+  return 0;
+}
+
+/* f32 -> OCP float8 e4m3fn (1-4-3, bias 7, max 448, no infinities), round to
+ * nearest even, for |x| <= 448 (callers clamp first).  Normal numbers:
+ * x = (1 + q/8) 2^e; subnormals: x = q 2^-9; in both cases the code is the
+ * rounded significand added to the exponent field, so a carry out of the
+ * mantissa lands in the exponent. */
+static inline uint8_t f32_to_e4m3fn(float x) {
+  uint32_t u;
+  memcpy(&u, &x, 4);
+  const uint8_t sign = (uint8_t)((u >> 24) & 0x80);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint8_t)(sign | 0x7f);
+  float a = fabsf(x);
+  int code;
+  if (a < 0.015625f) { /* below 2^-6: subnormal grid of 2^-9 */
+    code = (int)rintf(a * 512.0f);
+  } else {
+    int e;
+    float m = frexpf(a, &e); /* a = m 2^e, m in [0.5, 1) */
+    code = ((e - 1 + 7) << 3) + (int)rintf((m * 2.0f - 1.0f) * 8.0f);
+  }
+  if (code > 0x7e) code = 0x7e;
+  return (uint8_t)(sign | code);
+}
+
+/* Static-scale quantisation of a bf16 tensor, scaled_fp8_conversion<true> of
+ * csrc/quantization/fp8/common.cuh:38-56: x = f32(y) * (1.0f / scale), clamped to
+ * +-448, converted with round-to-nearest-even.  This is what the reference's
+ * unit test composes after the unquantised norm
+ * (tests/kernels/test_layernorm.py:113-131). */
+int tw_oracle_static_fp8_quant(uint8_t* out, const uint16_t* y, int64_t n, float scale) {
+  if (n < 0) return -1;
+  const float inv = 1.0f / scale;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    float x = bf16_to_f32(y[i]) * inv;
+    x = fmaxf(-448.0f, fminf(x, 448.0f));
+    out[i] = f32_to_e4m3fn(x);
   }
   return 0;
 }

@@ -57,6 +57,8 @@ def lib() -> ctypes.CDLL:
         L.tw_oracle_rms_norm.argtypes = [_u16p, _u16p, _u16p, i64, i64, f32, ci]
         L.tw_oracle_rms_norm_inplace.argtypes = [_u16p, _u16p, _u16p, i64, i64, f32, ci]
         L.tw_oracle_gemm_bf16_nt.argtypes = [_u16p, _u16p, _u16p, i64, i64, i64, ci]
+        L.tw_oracle_static_fp8_quant.argtypes = [ctypes.POINTER(ctypes.c_uint8), _u16p, i64, f32]
+        L.tw_oracle_static_fp8_quant.restype = ci
         for name in ("fused_add_rms_norm", "reduce_add_rms_norm", "rms_norm",
                      "rms_norm_inplace", "gemm_bf16_nt"):
             getattr(L, "tw_oracle_" + name).restype = ci
@@ -144,6 +146,15 @@ def gemm_bf16_nt(a, b, mode=ROUND_RNE):
     assert K == K2
     out = np.empty((M, N), np.uint16)
     _check(lib().tw_oracle_gemm_bf16_nt(_p(out), _p(a), _p(b), M, N, K, mode), "gemm")
+    return out
+
+
+def static_fp8_quant(y, scale):
+    """bf16 bit patterns -> e4m3fn codes (uint8): fp8_rne(clamp(f32(y) * (1/scale), +-448))."""
+    assert y.dtype == np.uint16 and y.flags["C_CONTIGUOUS"]
+    out = np.empty(y.shape, np.uint8)
+    _check(lib().tw_oracle_static_fp8_quant(out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)),
+                                            _p(y), y.size, scale), "static_fp8_quant")
     return out
 
 

@@ -296,3 +296,21 @@ def test_empty_input_is_a_no_op(oracle):
     x = np.zeros((0, 64), np.uint16)
     oracle.fused_add_rms_norm(x, x.copy(), np.zeros(64, np.uint16), 1e-5)
     assert oracle.rms_norm(x, np.zeros(64, np.uint16), 1e-5).shape == (0, 64)
+
+
+def test_fp8_quant_matches_torch_cast_on_every_bf16_pattern(oracle):
+    """Pins the e4m3fn conversion of the checker against an independent
+    implementation (torch's CPU cast), on all 65536 bf16 inputs and three scales."""
+    torch = pytest.importorskip("torch")
+    bits = np.arange(65536, dtype=np.uint16)
+    vals = torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16).float()
+    finite = torch.isfinite(vals).numpy()
+    for scale in (1.0, 0.01, 10.0, 0.37):
+        got = oracle.static_fp8_quant(bits, scale)
+        inv = torch.tensor(1.0, dtype=torch.float32) / torch.tensor(scale, dtype=torch.float32)
+        want = (vals * inv).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+        assert np.array_equal(got[finite], want[finite]), scale
+    # spot values: 448 saturates, ties go to even, subnormal grid is 2^-9
+    f = np.array([448.0, 1000.0, -1000.0, 0.0, 2 ** -9, 2 ** -10, 3 * 2 ** -10, 17.0, 19.0], np.float32)
+    got = oracle.static_fp8_quant(oracle.f32_to_bf16(f), 1.0)
+    assert list(got) == [0x7E, 0x7E, 0xFE, 0x00, 0x01, 0x00, 0x02, 0x58, 0x5A]

@@ -261,6 +261,84 @@ def reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
             _cap(MAX_CTAS), epsilon, _stream_ptr(out)))
 
 
+# ---------------------------------------------------------------------------
+# norm + static fp8 quantisation (vllm/_custom_ops.py rms_norm_static_fp8_quant /
+# fused_add_rms_norm_static_fp8_quant -> csrc/layernorm_quant_kernels.cu)
+# ---------------------------------------------------------------------------
+FP8_DTYPE = torch.float8_e4m3fn  # gfx950 implements the OCP formats
+
+
+def _check_fp8_out(out: torch.Tensor, like: torch.Tensor) -> None:
+    _require(out.is_cuda and out.device == like.device, f"result is on {out.device}, expected {like.device}")
+    if out.dtype != FP8_DTYPE:
+        raise NotImplementedError(f'"rms_norm_kernel_fp8_type" not implemented for \'{out.dtype}\'')
+    _require(out.is_contiguous() and out.shape == like.shape,
+             "result must be a contiguous fp8 tensor with the input's shape")
+
+
+def _check_scale(scale: torch.Tensor, device) -> None:
+    _require(isinstance(scale, torch.Tensor) and scale.is_cuda and scale.device == device,
+             "scale must be a tensor on the input's device")
+    _require(scale.dtype == torch.float32 and scale.numel() == 1, "scale must hold one float32 value")
+
+
+def rms_norm_static_fp8_quant(result: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,
+                              scale: torch.Tensor, epsilon: float) -> None:
+    code = _dtype_code("rms_norm_kernel_scalar_type", input)
+    _check_tensor("input", input, input.dtype, input.device)
+    _check_fp8_out(result, input)
+    T, H = _rows(input)
+    _check_weight(weight, H, input.dtype, input.device)
+    _check_scale(scale, input.device)
+    with _on_device(input):
+        _lib.check(_lib.lib().tw_rms_norm_static_fp8_quant(
+            result.data_ptr(), input.data_ptr(), weight.data_ptr(), scale.data_ptr(), T, H, epsilon,
+            code, _stream_ptr(input)))
+
+
+def fused_add_rms_norm_static_fp8_quant(result: torch.Tensor, input: torch.Tensor,
+                                        residual: torch.Tensor, weight: torch.Tensor,
+                                        scale: torch.Tensor, epsilon: float) -> None:
+    code = _dtype_code("fused_add_rms_norm_kernel_scalar_type", input)
+    _check_tensor("input", input, input.dtype, input.device)
+    _check_tensor("residual", residual, input.dtype, input.device)
+    _check_fp8_out(result, input)
+    T, H = _rows(input)
+    _require(residual.shape == input.shape, "input and residual must have the same shape")
+    _check_weight(weight, H, input.dtype, input.device)
+    _check_scale(scale, input.device)
+    with _on_device(input):
+        _lib.check(_lib.lib().tw_fused_add_rms_norm_static_fp8_quant(
+            result.data_ptr(), input.data_ptr(), residual.data_ptr(), weight.data_ptr(),
+            scale.data_ptr(), T, H, epsilon, code, _stream_ptr(input)))
+
+
+def reduce_add_rms_norm_static_fp8_quant(partials: Sequence[torch.Tensor], result: torch.Tensor,
+                                         residual: torch.Tensor, weight: torch.Tensor,
+                                         scale: torch.Tensor, epsilon: float,
+                                         MAX_CTAS: Optional[int] = None) -> None:
+    """result(fp8) <- quantised RMSNorm(sum_p partials[p] + residual) * weight; residual <- the sum."""
+    P = len(partials)
+    _require(1 <= P <= _lib.TW_MAX_PARTIALS,
+             f"number of partials {P} not in [1, {_lib.TW_MAX_PARTIALS}]")
+    _require_bf16("reduce_add_rms_norm_kernel", residual)
+    dev = residual.device
+    _check_tensor("residual", residual, torch.bfloat16, dev)
+    _check_fp8_out(result, residual)
+    T, H = _rows(residual)
+    for i, p in enumerate(partials):
+        _check_tensor(f"partials[{i}]", p, torch.bfloat16, dev)
+        _require(p.shape == residual.shape,
+                 f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(residual.shape)}")
+    _check_weight(weight, H, torch.bfloat16, dev)
+    _check_scale(scale, dev)
+    ptrs = (ctypes.c_void_p * P)(*[p.data_ptr() for p in partials])
+    with _on_device(residual):
+        _lib.check(_lib.lib().tw_reduce_add_rms_norm_static_fp8_quant(
+            ptrs, P, result.data_ptr(), residual.data_ptr(), weight.data_ptr(), scale.data_ptr(), T, H,
+            _cap(MAX_CTAS), epsilon, _stream_ptr(residual)))
+
+
 def gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
                  max_cus: Optional[int] = None) -> None:
     """out[M, N] <- a[M, K] @ b[N, K]^T (bf16, fp32 accumulate).  `out` may be a row
@@ -321,6 +399,13 @@ SCHEMAS = {
     "fused_rs_ln_cta":
         "fused_rs_ln_cta(Tensor! input, Tensor! residual, Tensor weight, int mcptr, "
         "int signal_pads, int rank, int world_size, int MAX_CTAS, float epsilon) -> ()",
+    # csrc/torch_bindings.cpp:199-213
+    "rms_norm_static_fp8_quant":
+        "rms_norm_static_fp8_quant(Tensor! result, Tensor input, Tensor weight, Tensor scale, "
+        "float epsilon) -> ()",
+    "fused_add_rms_norm_static_fp8_quant":
+        "fused_add_rms_norm_static_fp8_quant(Tensor! result, Tensor input, Tensor! residual, "
+        "Tensor weight, Tensor scale, float epsilon) -> ()",
 }
 
 _IMPLS = {
@@ -330,6 +415,8 @@ _IMPLS = {
     "fused_rs_ln_ag_cta": fused_rs_ln_ag_cta,
     "fused_add_rms_norm_cta": fused_add_rms_norm_cta,
     "fused_rs_ln_cta": fused_rs_ln_cta,
+    "rms_norm_static_fp8_quant": rms_norm_static_fp8_quant,
+    "fused_add_rms_norm_static_fp8_quant": fused_add_rms_norm_static_fp8_quant,
 }
 
 

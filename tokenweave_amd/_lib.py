@@ -39,6 +39,10 @@ PROTOTYPES = {
     "tw_fused_rs_ln_cta": [_vp, _vp, _vp, _u64, _i64, _ci, _ci, _ci, _f32, _i64, _i64, _vp],
     "tw_fused_rs_ln_ag_cta": [_vp, _vp, _vp, _u64, _i64, _ci, _ci, _ci, _f32, _i64, _i64, _vp],
     "tw_gemm_bf16_nt": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp],
+    "tw_rms_norm_static_fp8_quant": [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _ci, _vp],
+    "tw_fused_add_rms_norm_static_fp8_quant": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _ci, _vp],
+    "tw_reduce_add_rms_norm_static_fp8_quant": [ctypes.POINTER(_vp), _ci, _vp, _vp, _vp, _vp, _i64, _i64,
+                                                _ci, _f32, _vp],
     "tw_copy_bytes": [_vp, _vp, _i64, _vp],
 }
 

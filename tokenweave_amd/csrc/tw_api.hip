@@ -68,14 +68,14 @@ int tw_fused_add_rms_norm(void* input, void* residual, const void* weight, int64
   if (!residual && num_tokens > 0)
     return tw::set_error(TW_ERR_INVALID_ARGUMENT, "fused_add_rms_norm: residual is null");
   const void* parts[1] = {input};
-  return tw::run_row_norm("fused_add_rms_norm", parts, 1, input, residual, nullptr, weight,
+  return tw::run_row_norm("fused_add_rms_norm", parts, 1, input, residual, nullptr, weight, nullptr,
                           num_tokens, hidden_size, epsilon, dtype, 0, false, stream);
 }
 
 int tw_rms_norm(void* out, const void* input, const void* weight, int64_t num_tokens,
                 int64_t hidden_size, float epsilon, int dtype, void* stream) {
   const void* parts[1] = {input};
-  return tw::run_row_norm("rms_norm", parts, 1, out, nullptr, nullptr, weight, num_tokens,
+  return tw::run_row_norm("rms_norm", parts, 1, out, nullptr, nullptr, weight, nullptr, num_tokens,
                           hidden_size, epsilon, dtype, 0, false, stream);
 }
 
@@ -86,7 +86,7 @@ int tw_rms_norm_inplace(void* out, void* input, const void* weight, int64_t num_
   if (out == input && num_tokens > 0)
     return tw::set_error(TW_ERR_INVALID_ARGUMENT, "rms_norm_inplace: out must not alias input");
   const void* parts[1] = {input};
-  return tw::run_row_norm("rms_norm_inplace", parts, 1, input, nullptr, out, weight, num_tokens,
+  return tw::run_row_norm("rms_norm_inplace", parts, 1, input, nullptr, out, weight, nullptr, num_tokens,
                           hidden_size, epsilon, dtype, 0, false, stream);
 }
 
@@ -96,7 +96,7 @@ int tw_fused_add_rms_norm_cta(void* input, void* residual, const void* weight,
   if (!residual && num_tokens > 0)
     return tw::set_error(TW_ERR_INVALID_ARGUMENT, "fused_add_rms_norm_cta: residual is null");
   const void* parts[1] = {input};
-  return tw::run_row_norm("fused_add_rms_norm_cta", parts, 1, input, residual, nullptr, weight,
+  return tw::run_row_norm("fused_add_rms_norm_cta", parts, 1, input, residual, nullptr, weight, nullptr,
                           num_tokens, hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true, stream);
 }
 
@@ -106,7 +106,7 @@ int tw_reduce_add_rms_norm(const void* const* partials, int num_partials, void* 
   if (!residual && num_tokens > 0)
     return tw::set_error(TW_ERR_INVALID_ARGUMENT, "reduce_add_rms_norm: residual is null");
   return tw::run_row_norm("reduce_add_rms_norm", partials, num_partials, y, residual, nullptr,
-                          weight, num_tokens, hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true,
+                          weight, nullptr, num_tokens, hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true,
                           stream);
 }
 
@@ -119,7 +119,7 @@ int tw_fused_rs_ln_cta(void* input, void* residual, const void* weight, uint64_t
   if (rc != TW_OK) return rc;
   if (!residual && num_tokens > 0)
     return tw::set_error(TW_ERR_INVALID_ARGUMENT, "fused_rs_ln_cta: residual is null");
-  return tw::run_row_norm("fused_rs_ln_cta", parts, world_size, input, residual, nullptr, weight,
+  return tw::run_row_norm("fused_rs_ln_cta", parts, world_size, input, residual, nullptr, weight, nullptr,
                           num_tokens, hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true, stream);
 }
 
@@ -133,8 +133,42 @@ int tw_fused_rs_ln_ag_cta(void* input, void* residual, const void* weight, uint6
   if (!residual && num_tokens > 0)
     return tw::set_error(TW_ERR_INVALID_ARGUMENT, "fused_rs_ln_ag_cta: residual is null");
   return tw::run_row_norm("fused_rs_ln_ag_cta", parts, world_size, input, residual, nullptr,
-                          weight, num_tokens, hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true,
+                          weight, nullptr, num_tokens, hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true,
                           stream);
+}
+
+int tw_rms_norm_static_fp8_quant(void* out, const void* input, const void* weight,
+                                 const float* scale, int64_t num_tokens, int64_t hidden_size,
+                                 float epsilon, int dtype, void* stream) {
+  if (!scale && num_tokens > 0)
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "rms_norm_static_fp8_quant: scale is null");
+  const void* parts[1] = {input};
+  return tw::run_row_norm("rms_norm_static_fp8_quant", parts, 1, out, nullptr, nullptr, weight, scale,
+                          num_tokens, hidden_size, epsilon, dtype, 0, false, stream);
+}
+
+int tw_fused_add_rms_norm_static_fp8_quant(void* out, const void* input, void* residual,
+                                           const void* weight, const float* scale,
+                                           int64_t num_tokens, int64_t hidden_size, float epsilon,
+                                           int dtype, void* stream) {
+  if ((!scale || !residual) && num_tokens > 0)
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT,
+                         "fused_add_rms_norm_static_fp8_quant: scale or residual is null");
+  const void* parts[1] = {input};
+  return tw::run_row_norm("fused_add_rms_norm_static_fp8_quant", parts, 1, out, residual, nullptr,
+                          weight, scale, num_tokens, hidden_size, epsilon, dtype, 0, false, stream);
+}
+
+int tw_reduce_add_rms_norm_static_fp8_quant(const void* const* partials, int num_partials, void* out,
+                                            void* residual, const void* weight, const float* scale,
+                                            int64_t num_tokens, int64_t hidden_size, int max_ctas,
+                                            float epsilon, void* stream) {
+  if ((!scale || !residual) && num_tokens > 0)
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT,
+                         "reduce_add_rms_norm_static_fp8_quant: scale or residual is null");
+  return tw::run_row_norm("reduce_add_rms_norm_static_fp8_quant", partials, num_partials, out,
+                          residual, nullptr, weight, scale, num_tokens, hidden_size, epsilon,
+                          TW_DTYPE_BF16, max_ctas, true, stream);
 }
 
 int tw_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {

@@ -16,8 +16,8 @@ int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3
 int device_compute_units();
 
 int run_row_norm(const char* what, const void* const* partials, int np, void* y,
-                 void* residual, void* copy_out, const void* weight, int64_t T,
-                 int64_t H, float eps, int dtype, int max_ctas, bool require_vec,
+                 void* residual, void* copy_out, const void* weight, const float* quant_scale,
+                 int64_t T, int64_t H, float eps, int dtype, int max_ctas, bool require_vec,
                  void* stream);
 
 int run_copy16(void* dst, const void* src, int64_t nbytes, void* stream);

@@ -2,11 +2,11 @@
 //
 // One workgroup owns one token row at a time and keeps the whole row in
 // registers between the sum-of-squares reduction and the normalised store:
-// every byte is read once and written once.  At hidden size 8192 and 64 rows or
+// every byte is read once and written once.  At hidden size 8192 and 224 rows or
 // more a workgroup is 256 lanes (4 waves), each lane owning four 16-byte vectors
 // (8 bf16 each) of the row in every buffer; it issues its 4*(P+1) loads back to
 // back, so a row keeps (P+1)*16 KiB of HBM reads in flight.  With fewer rows a
-// row is spread over 1024 lanes, one vector each.
+// row is spread over 512 or 1024 lanes (two or one vector each).
 //
 // Memory policy, measured on MI355X with operands rotated through > 1 GiB:
 //   * partial and residual loads carry the non-temporal bit: the data is used
@@ -166,6 +166,27 @@ __device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t d, uint32_t off) 
   return make_uint4(t.x, t.y, t.z, t.w);
 }
 
+// Static-scale fp8 (OCP e4m3fn) quantisation of four values: multiply by the
+// inverted scale, clamp to the finite range, round to nearest even
+// (v_cvt_pk_fp8_f32).  scaled_fp8_conversion<true> of the reference
+// (csrc/quantization/fp8/common.cuh:38-56).
+constexpr float kFp8Max = 448.0f;
+__device__ __forceinline__ uint32_t quant4_fp8(float a, float b, float c, float d, float scale_inv) {
+  a = fmaxf(-kFp8Max, fminf(a * scale_inv, kFp8Max));
+  b = fmaxf(-kFp8Max, fminf(b * scale_inv, kFp8Max));
+  c = fmaxf(-kFp8Max, fminf(c * scale_inv, kFp8Max));
+  d = fmaxf(-kFp8Max, fminf(d * scale_inv, kFp8Max));
+  int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+  return (uint32_t)r;
+}
+
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store8(__amdgpu_buffer_rsrc_t d, uint32_t off, uint32_t lo, uint32_t hi) {
+  u32x2_t t = {lo, hi};
+  __builtin_amdgcn_raw_buffer_store_b64(t, d, off, 0, kStoreStream);
+}
+
 __device__ __forceinline__ void store16(__amdgpu_buffer_rsrc_t d, uint32_t off, const uint4& v) {
   u32x4_t t = {v.x, v.y, v.z, v.w};
   __builtin_amdgcn_raw_buffer_store_b128(t, d, off, 0, kStoreStream);
@@ -182,10 +203,11 @@ __device__ __forceinline__ void store16(__amdgpu_buffer_rsrc_t d, uint32_t off, 
 // y may alias any partial: a lane stores y only to vector slots it has already
 // read in every buffer.  blockDim.x must be a multiple of 64.
 // ---------------------------------------------------------------------------
-template <int NP, int VPT, int MAXNT, bool HAS_RES, bool COPY>
+template <int NP, int VPT, int MAXNT, bool HAS_RES, bool COPY, bool FP8>
 __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
     PartialPtrs parts, int np_rt, void* y_out, void* residual, void* copy_out,
-    const void* __restrict__ weight, float eps, int num_tokens, int vec_per_row, float hidden) {
+    const void* __restrict__ weight, const float* __restrict__ quant_scale, float eps,
+    int num_tokens, int vec_per_row, float hidden) {
   __shared__ float slots[2][kMaxChunks];
   const int nt = blockDim.x;
   const int nwaves = nt >> 6;
@@ -202,7 +224,7 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
   for (int row = blockIdx.x; row < num_tokens; row += gridDim.x, phase ^= 1) {
     float s[VPT][8];
     uint4 first[VPT];
-    const __amdgpu_buffer_rsrc_t dr = row_desc(HAS_RES ? residual : y_out, row, row_bytes);
+    const __amdgpu_buffer_rsrc_t dr = row_desc(HAS_RES ? residual : parts.p[0], row, row_bytes);
 
     if (NP > 0 && (VPT <= 2 || MAXNT <= 256)) {
       // Issue every load of the row before the first use.  (Four vectors per lane
@@ -279,7 +301,11 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
     const float total = row_sum_chunks<VPT>(ss, slots[phase], nwaves, nchunks);
     const float inv = inv_rms(total, hidden, eps);
 
-    const __amdgpu_buffer_rsrc_t dy = row_desc(y_out, row, row_bytes);
+    // bf16 output: 16 bytes per vector; fp8 output: the bf16 result quantised, 8 bytes
+    // per vector in rows of half the size.
+    const __amdgpu_buffer_rsrc_t dy = row_desc(y_out, row, FP8 ? row_bytes / 2 : row_bytes);
+    float scale_inv = 1.0f;
+    if (FP8) scale_inv = 1.0f / *quant_scale;
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       float r[8], w[8];
@@ -290,7 +316,14 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
       o.y = pack_bf16(r[2] * inv * w[2], r[3] * inv * w[3]);
       o.z = pack_bf16(r[4] * inv * w[4], r[5] * inv * w[5]);
       o.w = pack_bf16(r[6] * inv * w[6], r[7] * inv * w[7]);
-      store16(dy, off[k], o);
+      if (FP8) {
+        float y[8];
+        unpack8(o, y);
+        store8(dy, off[k] / 2, quant4_fp8(y[0], y[1], y[2], y[3], scale_inv),
+               quant4_fp8(y[4], y[5], y[6], y[7], scale_inv));
+      } else {
+        store16(dy, off[k], o);
+      }
     }
   }
 }
@@ -317,14 +350,17 @@ template <> struct Elem<float> {
   static __device__ __forceinline__ float round(float f) { return f; }
 };
 
-template <typename T, bool HAS_RES, bool COPY>
+template <typename T, bool HAS_RES, bool COPY, bool FP8>
 __global__ __launch_bounds__(1024) void row_norm_elem_kernel(
-    PartialPtrs parts, int np, T* y_out, T* residual, T* copy_out,
-    const T* __restrict__ weight, float eps, int num_tokens, int hidden_size) {
+    PartialPtrs parts, int np, void* y_out, T* residual, T* copy_out,
+    const T* __restrict__ weight, const float* __restrict__ quant_scale, float eps,
+    int num_tokens, int hidden_size) {
   __shared__ float slots[2][16];
   const int tid = threadIdx.x;
   const int nt = blockDim.x;
   const int nwaves = nt >> 6;
+  float scale_inv = 1.0f;
+  if (FP8) scale_inv = 1.0f / *quant_scale;
   int phase = 0;
   for (int row = blockIdx.x; row < num_tokens; row += gridDim.x, phase ^= 1) {
     const size_t base = (size_t)row * hidden_size;
@@ -346,7 +382,14 @@ __global__ __launch_bounds__(1024) void row_norm_elem_kernel(
       const T raw = src[base + j];
       const float r = Elem<T>::load(&raw);
       if (COPY) copy_out[base + j] = raw;
-      y_out[base + j] = Elem<T>::round(r * inv * Elem<T>::load(weight + j));
+      const T y = Elem<T>::round(r * inv * Elem<T>::load(weight + j));
+      if (FP8) {
+        const float q = fmaxf(-kFp8Max, fminf(Elem<T>::load(&y) * scale_inv, kFp8Max));
+        static_cast<uint8_t*>(y_out)[base + j] =
+            (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(q, q, 0, false) & 0xff);
+      } else {
+        static_cast<T*>(y_out)[base + j] = y;
+      }
     }
   }
 }
@@ -365,13 +408,15 @@ static int default_grid(int64_t num_tokens) {
 }
 
 // Workgroup shape for rows of V 16-byte vectors and T rows.  Results do not
-// depend on the shape (row_sum_chunks), so it is chosen for speed alone:
-//   * few rows (T < 64): as many lanes per row as the row has vectors (up to
-//     1024), one or two vectors each — the shortest path from launch to the last
-//     store when the call is latency bound;
-//   * many rows: four vectors per lane in workgroups of at most 256 lanes, every
-//     load of the row in flight at once (the fastest shape measured from 256 to
-//     8192 rows at hidden sizes 6144 and 8192);
+// depend on the shape (row_sum_chunks), so it is chosen for speed alone, from
+// sweeps at hidden size 8192 / 6144 with cold operands:
+//   * T < 48: as many lanes per row as the row has vectors (up to 1024), one
+//     vector each — the shortest path from launch to the last store when the
+//     call is latency bound;
+//   * 48 <= T < 224: two vectors per lane (512 lanes at hidden size 8192), 3-5 %
+//     ahead of both neighbours while there are fewer rows than compute units;
+//   * T >= 224: four vectors per lane in workgroups of at most 256 lanes, every
+//     load of the row in flight at once (fastest from 256 to 8192 rows);
 //   * rows longer than 1024 vectors: two vectors per lane up to 2048 vectors, four
 //     up to 4096 (one partial at a time).  Longer rows take the element-wise kernel.
 struct VecShape { int vpt, nt, maxnt; };
@@ -379,7 +424,8 @@ struct VecShape { int vpt, nt, maxnt; };
 static bool vec_shape(int V, int64_t T, VecShape* sh) {
   int vpt, maxnt = 1024;
   if (V <= 1024) {
-    if (T < 64 || V < 256) vpt = 1;
+    if (T < 48 || V < 128) vpt = 1;
+    else if (T < 224 || V < 256) vpt = 2;
     else { vpt = 4; maxnt = 256; }
   } else if (V <= 2048) vpt = 2;
   else if (V <= 4096) vpt = 4;
@@ -391,17 +437,30 @@ static bool vec_shape(int V, int64_t T, VecShape* sh) {
   return true;
 }
 
-template <int NP, bool HAS_RES, bool COPY>
-static int launch_vec_vpt(const PartialPtrs& parts, int np, void* y, void* residual,
-                          void* copy_out, const void* weight, int64_t T, int64_t H,
-                          float eps, int grid, hipStream_t stream) {
-  const int V = (int)(H / 8);
+struct RowNormArgs {
+  PartialPtrs parts;
+  int np;
+  void* y;
+  void* residual;
+  void* copy_out;
+  const void* weight;
+  const float* quant_scale;  // non-null: y is fp8 (e4m3fn), quantised with this device scalar
+  int64_t T, H;
+  float eps;
+  int grid;
+  hipStream_t stream;
+};
+
+template <int NP, bool HAS_RES, bool COPY, bool FP8>
+static int launch_vec(const RowNormArgs& a) {
+  const int V = (int)(a.H / 8);
   VecShape sh;
-  if (!vec_shape(V, T, &sh)) return 1;  // caller falls back to the element-wise kernel
-  dim3 g(grid), b(sh.nt);
-#define TW_LAUNCH(VPT, MAXNT)                                                                  \
-  hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, MAXNT, HAS_RES, COPY>), g, b, 0, stream,   \
-                     parts, np, y, residual, copy_out, weight, eps, (int)T, V, (float)H)
+  if (!vec_shape(V, a.T, &sh)) return 1;  // caller falls back to the element-wise kernel
+  dim3 g(a.grid), b(sh.nt);
+#define TW_LAUNCH(VPT, MAXNT)                                                                    \
+  hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, MAXNT, HAS_RES, COPY, FP8>), g, b, 0,        \
+                     a.stream, a.parts, a.np, a.y, a.residual, a.copy_out, a.weight,             \
+                     a.quant_scale, a.eps, (int)a.T, V, (float)a.H)
   if (sh.vpt == 1) TW_LAUNCH(1, 1024);
   else if (sh.vpt == 2) TW_LAUNCH(2, 1024);
   else if (sh.maxnt == 256) TW_LAUNCH(4, 256);
@@ -410,20 +469,29 @@ static int launch_vec_vpt(const PartialPtrs& parts, int np, void* y, void* resid
   return 0;
 }
 
+// mode: residual given -> add + write back; copy_out given -> rms_norm_inplace;
+// neither -> rms_norm.  Only the P = 1 kernels exist without a residual.
+template <int NP>
+static int launch_vec_mode(const RowNormArgs& a) {
+  const bool fp8 = a.quant_scale != nullptr;
+  if (a.residual) return fp8 ? launch_vec<NP, true, false, true>(a) : launch_vec<NP, true, false, false>(a);
+  if (NP != 1) return 1;
+  if (a.copy_out) return fp8 ? 1 : launch_vec<1, false, true, false>(a);
+  return fp8 ? launch_vec<1, false, false, true>(a) : launch_vec<1, false, false, false>(a);
+}
+
 template <typename T>
-static void launch_elem_t(const PartialPtrs& parts, int np, void* y, void* residual,
-                          void* copy_out, const void* weight, int64_t Tn, int64_t H,
-                          float eps, int grid, hipStream_t stream) {
-  int nt = H < 1024 ? (int)((H + 63) / 64) * 64 : 1024;
-  dim3 g(grid), b(nt);
-#define TW_LAUNCH(HAS_RES, COPY)                                                     \
-  hipLaunchKernelGGL((row_norm_elem_kernel<T, HAS_RES, COPY>), g, b, 0, stream, parts, \
-                     np, static_cast<T*>(y), static_cast<T*>(residual),               \
-                     static_cast<T*>(copy_out), static_cast<const T*>(weight), eps,   \
-                     (int)Tn, (int)H)
-  if (residual) TW_LAUNCH(true, false);
-  else if (copy_out) TW_LAUNCH(false, true);
-  else TW_LAUNCH(false, false);
+static void launch_elem(const RowNormArgs& a) {
+  int nt = a.H < 1024 ? (int)((a.H + 63) / 64) * 64 : 1024;
+  dim3 g(a.grid), b(nt);
+#define TW_LAUNCH(HAS_RES, COPY, FP8)                                                            \
+  hipLaunchKernelGGL((row_norm_elem_kernel<T, HAS_RES, COPY, FP8>), g, b, 0, a.stream, a.parts,  \
+                     a.np, a.y, static_cast<T*>(a.residual), static_cast<T*>(a.copy_out),        \
+                     static_cast<const T*>(a.weight), a.quant_scale, a.eps, (int)a.T, (int)a.H)
+  const bool fp8 = a.quant_scale != nullptr;
+  if (a.residual) { if (fp8) TW_LAUNCH(true, false, true); else TW_LAUNCH(true, false, false); }
+  else if (a.copy_out) TW_LAUNCH(false, true, false);
+  else { if (fp8) TW_LAUNCH(false, false, true); else TW_LAUNCH(false, false, false); }
 #undef TW_LAUNCH
 }
 
@@ -435,11 +503,12 @@ static int finish_launch(const char* what) {
 }
 
 // Shared by every entry point.  residual == nullptr: no residual add;
-// copy_out != nullptr: rms_norm_inplace.  require_vec: refuse instead of
-// falling back to the element-wise kernel (the *_cta contract).
+// copy_out != nullptr: rms_norm_inplace; quant_scale != nullptr: y is fp8.
+// require_vec: refuse instead of falling back to the element-wise kernel (the
+// *_cta contract).
 int run_row_norm(const char* what, const void* const* partials, int np, void* y,
-                 void* residual, void* copy_out, const void* weight, int64_t T,
-                 int64_t H, float eps, int dtype, int max_ctas, bool require_vec,
+                 void* residual, void* copy_out, const void* weight, const float* quant_scale,
+                 int64_t T, int64_t H, float eps, int dtype, int max_ctas, bool require_vec,
                  void* stream_v) {
   if (np < 1 || np > TW_MAX_PARTIALS)
     return set_error(TW_ERR_INVALID_ARGUMENT, "%s: number of partials %d not in [1, %d]", what, np,
@@ -452,16 +521,19 @@ int run_row_norm(const char* what, const void* const* partials, int np, void* y,
   if (T == 0) return TW_OK;
   if (!y || !weight || !partials)
     return set_error(TW_ERR_INVALID_ARGUMENT, "%s: null pointer argument", what);
-  PartialPtrs parts = {};
+  if (quant_scale && copy_out)
+    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: fp8 output is not defined for the in-place op", what);
+  RowNormArgs a = {};
   bool aligned = aligned16(y) && aligned16(weight) && (!residual || aligned16(residual)) &&
                  (!copy_out || aligned16(copy_out));
   for (int p = 0; p < np; ++p) {
     if (!partials[p])
       return set_error(TW_ERR_INVALID_ARGUMENT, "%s: partial %d is a null pointer", what, p);
-    parts.p[p] = partials[p];
+    a.parts.p[p] = partials[p];
     aligned = aligned && aligned16(partials[p]);
   }
-  const bool vec_ok = aligned && (H % 8 == 0);
+  // fp8 rows are H bytes: H % 16 keeps every row of the output 16-byte aligned too
+  const bool vec_ok = aligned && (H % 8 == 0) && (!quant_scale || H % 16 == 0);
   if (require_vec && (!vec_ok || dtype != TW_DTYPE_BF16)) {
     if (dtype != TW_DTYPE_BF16)
       return set_error(TW_ERR_DTYPE, "%s: only bf16 is supported", what);
@@ -472,38 +544,35 @@ int run_row_norm(const char* what, const void* const* partials, int np, void* y,
   }
   int grid = max_ctas > 0 ? max_ctas : default_grid(T);
   if (grid > T) grid = (int)T;
-  hipStream_t stream = static_cast<hipStream_t>(stream_v);
+  a.np = np;
+  a.y = y;
+  a.residual = residual;
+  a.copy_out = copy_out;
+  a.weight = weight;
+  a.quant_scale = quant_scale;
+  a.T = T;
+  a.H = H;
+  a.eps = eps;
+  a.grid = grid;
+  a.stream = static_cast<hipStream_t>(stream_v);
 
   if (vec_ok && dtype == TW_DTYPE_BF16) {
     int fell = 1;
-#define TW_MODE(NP)                                                                       \
-  (residual ? launch_vec_vpt<NP, true, false>(parts, np, y, residual, nullptr, weight, T, \
-                                              H, eps, grid, stream)                       \
-   : copy_out ? launch_vec_vpt<NP, false, true>(parts, np, y, nullptr, copy_out, weight,  \
-                                                T, H, eps, grid, stream)                  \
-              : launch_vec_vpt<NP, false, false>(parts, np, y, nullptr, nullptr, weight,  \
-                                                 T, H, eps, grid, stream))
     switch (np) {
-      case 1: fell = TW_MODE(1); break;
-      case 2: fell = residual ? launch_vec_vpt<2, true, false>(parts, np, y, residual, nullptr, weight, T, H, eps, grid, stream) : 1; break;
-      case 4: fell = residual ? launch_vec_vpt<4, true, false>(parts, np, y, residual, nullptr, weight, T, H, eps, grid, stream) : 1; break;
-      case 8: fell = residual ? launch_vec_vpt<8, true, false>(parts, np, y, residual, nullptr, weight, T, H, eps, grid, stream) : 1; break;
-      default: fell = residual ? launch_vec_vpt<0, true, false>(parts, np, y, residual, nullptr, weight, T, H, eps, grid, stream) : 1; break;
+      case 1: fell = launch_vec_mode<1>(a); break;
+      case 2: fell = launch_vec_mode<2>(a); break;
+      case 4: fell = launch_vec_mode<4>(a); break;
+      case 8: fell = launch_vec_mode<8>(a); break;
+      default: fell = launch_vec_mode<0>(a); break;
     }
-#undef TW_MODE
     if (fell == 0) return finish_launch(what);
-    // rows longer than 4 vectors per lane: the element-wise kernel below
+    // rows longer than 4 vectors per lane (or a mode without a vector kernel):
+    // the element-wise kernel below
   }
   switch (dtype) {
-    case TW_DTYPE_BF16:
-      launch_elem_t<__bf16>(parts, np, y, residual, copy_out, weight, T, H, eps, grid, stream);
-      break;
-    case TW_DTYPE_F16:
-      launch_elem_t<_Float16>(parts, np, y, residual, copy_out, weight, T, H, eps, grid, stream);
-      break;
-    default:
-      launch_elem_t<float>(parts, np, y, residual, copy_out, weight, T, H, eps, grid, stream);
-      break;
+    case TW_DTYPE_BF16: launch_elem<__bf16>(a); break;
+    case TW_DTYPE_F16: launch_elem<_Float16>(a); break;
+    default: launch_elem<float>(a); break;
   }
   return finish_launch(what);
 }

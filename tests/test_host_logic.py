@@ -156,3 +156,21 @@ def test_workload_generation_is_seeded_and_shaped():
     assert not torch.equal(a.staging, c.staging)
     g = wl.make_gemm_inputs(16, 32, 64, "cpu")
     assert g.a.shape == (16, 64) and g.b.shape == (32, 64) and abs(g.b.float().std() - 0.02) < 0.005
+
+
+def test_weave_config_table_and_plan():
+    cfg = tw.load_config()          # packaged llama_config_8.json, same layout as the reference's tables
+    assert cfg is tw.load_config()  # cached per path (tokenweave_utils.py:10)
+    assert all(isinstance(k, int) for k in cfg) and 1024 in cfg
+    for entry in cfg.values():
+        assert {"attention_ctas", "mlp_ctas", "split_offset", "gemm_cus"} <= set(entry)
+    assert tw.select_config(cfg, 1500) is cfg[1024]      # closest length, llama.py:516
+    assert tw.select_config(cfg, 1537) is cfg[2048]
+    assert tw.weave_plan(1023, cfg) is None              # below the weave threshold: fuse only
+    plan = tw.weave_plan(4096, cfg)
+    off = cfg[4096]["split_offset"]
+    assert plan["split_size"] == 2048 + off and plan["rest_size"] == 4096 - plan["split_size"]
+    assert plan["gemm_cus"] == cfg[4096]["gemm_cus"]
+    table = {1024: {"attention_ctas": 8, "mlp_ctas": 4, "split_offset": 256}}
+    assert tw.weave_plan(1100, table) == {"split_size": 896, "rest_size": 204, "attention_ctas": 8,
+                                          "mlp_ctas": 4, "gemm_cus": 0}

@@ -8,8 +8,9 @@ reference's op shims (``vllm/_custom_ops.py:176-221``), its ``RMSNorm`` layer
 from . import _custom_ops as ops  # noqa: F401
 from .layernorm import RMSNorm  # noqa: F401
 from .tokenweave_utils import (PartialsBuffer, fused_allreduce_layernorm,  # noqa: F401
-                               shard_bounds, tokenweave_split_size, weave_norm_gemm)
+                               load_config, select_config, shard_bounds, tokenweave_split_size,
+                               weave_norm_gemm, weave_plan)
 
 __all__ = ["ops", "RMSNorm", "PartialsBuffer", "fused_allreduce_layernorm", "shard_bounds",
-           "tokenweave_split_size", "weave_norm_gemm"]
+           "tokenweave_split_size", "weave_norm_gemm", "load_config", "select_config", "weave_plan"]
 __version__ = "0.1.0"

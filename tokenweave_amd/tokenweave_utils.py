@@ -9,12 +9,54 @@ stream while the other split's row-parallel GEMM runs on the current stream.
 """
 from __future__ import annotations
 
-from typing import Any, Callable, Optional, Tuple
+import json
+import os
+from functools import lru_cache
+from typing import Any, Callable, Dict, Optional, Tuple
 
 import torch
 
 from . import _custom_ops as ops
 from .layernorm import RMSNorm
+
+
+@lru_cache(maxsize=None)
+def load_config(config_path: str = "tokenweave_configs/llama_config_8.json") -> Dict[int, Dict[str, int]]:
+    """Per-model weave table: token count -> {"attention_ctas", "mlp_ctas", "split_offset",
+    "gemm_cus"}.  Same file layout and loader contract as the reference
+    (tokenweave_utils.py:10-21, vllm/tokenweave_configs/*.json): JSON object with
+    string token-count keys, returned with integer keys and cached per path.
+    `*_ctas` is the MAX_CTAS given to the fused norm of the attention / MLP stage (0 =
+    one workgroup per row), `gemm_cus` the compute-unit budget of the GEMM it overlaps
+    with — the knob that matters on MI355X, where a GEMM workgroup and a norm workgroup
+    cannot share a compute unit.  Relative paths resolve against this package."""
+    base_dir = os.path.dirname(os.path.abspath(__file__))
+    full_path = config_path if os.path.isabs(config_path) else os.path.normpath(
+        os.path.join(base_dir, config_path))
+    with open(full_path, "r") as f:
+        data = json.load(f)
+    return {int(k): v for k, v in data.items()}
+
+
+def select_config(config: Dict[int, Dict[str, int]], num_tokens: int) -> Dict[str, int]:
+    """The entry whose token count is closest to num_tokens
+    (vllm/model_executor/models/llama.py:516-517); ties go to the smaller count."""
+    closest = min(sorted(config), key=lambda k: abs(k - num_tokens))
+    return config[closest]
+
+
+def weave_plan(num_tokens: int, config: Dict[int, Dict[str, int]],
+               threshold: int = 1024) -> Optional[Dict[str, int]]:
+    """What the model forward decides per batch (llama.py:509-521): below `threshold`
+    tokens no weave (fuse only) -> None; otherwise the split point and the budgets of
+    the closest table entry."""
+    if num_tokens < threshold:
+        return None
+    entry = select_config(config, num_tokens)
+    split = min(tokenweave_split_size(num_tokens, entry.get("split_offset", 0)), num_tokens)
+    return {"split_size": split, "rest_size": num_tokens - split,
+            "attention_ctas": entry.get("attention_ctas", 0), "mlp_ctas": entry.get("mlp_ctas", 0),
+            "gemm_cus": entry.get("gemm_cus", 0)}
 
 
 class PartialsBuffer:

@@ -1,0 +1,119 @@
+"""Measures, on the GPU it runs on, the weave budgets for one model shape and
+writes a table in the layout `load_config` reads.
+
+    python -m tokenweave_amd.tune_weave --hidden 8192 --k 1024 --world-size 8 \\
+        --tokens 1024 2048 4096 8192 --out tokenweave_amd/tokenweave_configs/llama_config_8.json
+
+For every token count N and split offset it times the stage the reference overlaps
+(tokenweave_utils.py:236-260): the row-parallel GEMM [split, K] x [hidden, K]^T of one
+token split on the current stream while the fused P-partial norm of the other split
+runs on a second stream, over a grid of GEMM compute-unit budgets and norm grid caps,
+and keeps the fastest.  The role of artifact/configs_generator/generator.py in the
+reference, which picks the minimum-latency row of its benchmark sweep.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import sys
+
+import torch
+
+from . import _custom_ops as ops
+from . import _lib
+from . import workloads as wl
+from .tokenweave_utils import tokenweave_split_size
+
+
+def time_stage(L, gemm_args, norm_sets, gemm_cus, norm_ctas, steps=40):
+    main_s, side_s = torch.cuda.Stream(), torch.cuda.Stream()
+    pm, ps = ctypes.c_void_p(main_s.cuda_stream), ctypes.c_void_p(side_s.cuda_stream)
+    out, a, b, M, N, K = gemm_args
+
+    def stage(i):
+        before = torch.cuda.Event()
+        before.record(main_s)
+        rc = L.tw_gemm_bf16_nt(out, a, b, M, N, K, N, gemm_cus, pm)
+        side_s.wait_event(before)
+        ptrs, P, y, r, w, T, H, eps = norm_sets[i % len(norm_sets)]
+        rc |= L.tw_reduce_add_rms_norm(ptrs, P, y, r, w, T, H, norm_ctas, eps, ps)
+        main_s.wait_stream(side_s)
+        if rc:
+            raise RuntimeError(_lib.last_error())
+
+    with torch.cuda.stream(main_s):
+        for i in range(5):
+            stage(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(main_s)
+        for i in range(steps):
+            stage(i)
+        e1.record(main_s)
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / steps
+
+
+def tune(hidden, k, world_size, tokens, offsets, device="cuda:0", log=print):
+    L = _lib.lib()
+    cus = ops.num_compute_units(device)
+    gemm_grid = sorted({0} | {int(cus * f) // 8 * 8 for f in (0.5, 0.5625, 0.625, 0.6875, 0.75, 0.875)})
+    norm_grid = (0, cus // 2, cus // 4 * 3)
+    table = {}
+    for n in tokens:
+        best = None
+        for off in offsets:
+            split = min(tokenweave_split_size(n, off), n)
+            rest = n - split
+            if split == 0 or rest == 0:
+                continue
+            g = wl.make_gemm_inputs(split, hidden, k, device)
+            out = torch.empty((split, hidden), dtype=torch.bfloat16, device=device)
+            cfg = wl.NormConfig("tune", P=world_size, T=rest, H=hidden, eps=1e-5, seed=77,
+                                partial_std=world_size ** -0.5)
+            nsets = max(2, min(8, (1 << 31) // cfg.bytes))
+            keep, sets = [], []
+            for i in range(nsets):
+                inp = wl.make_norm_inputs(cfg, device, seed_offset=i)
+                ops.reduce_add_rms_norm(inp.partials, inp.partials[0], inp.residual, inp.weight, cfg.eps)
+                ptrs = (ctypes.c_void_p * cfg.P)(*[p.data_ptr() for p in inp.partials])
+                keep.append((inp, ptrs))
+                sets.append((ptrs, cfg.P, inp.partials[0].data_ptr(), inp.residual.data_ptr(),
+                             inp.weight.data_ptr(), cfg.T, cfg.H, cfg.eps))
+            ops.gemm_bf16_nt(out, g.a, g.b)
+            gargs = (out.data_ptr(), g.a.data_ptr(), g.b.data_ptr(), split, hidden, k)
+            for gc in gemm_grid:
+                for nc in norm_grid:
+                    us = time_stage(L, gargs, sets, gc, nc)
+                    if best is None or us < best[0]:
+                        best = (us, off, gc, nc)
+            del keep, sets, g, out
+            torch.cuda.empty_cache()
+        us, off, gc, nc = best
+        log(f"tokens={n}: best stage {us:.1f} us with split_offset={off} gemm_cus={gc} norm_ctas={nc}")
+        table[str(n)] = {"attention_ctas": nc, "mlp_ctas": nc, "split_offset": off, "gemm_cus": gc}
+    return table
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--hidden", type=int, default=8192)
+    ap.add_argument("--k", type=int, default=1024, help="inner dimension of the row-parallel GEMM (per rank)")
+    ap.add_argument("--world-size", type=int, default=8)
+    ap.add_argument("--tokens", type=int, nargs="+", default=[1024, 2048, 4096, 8192])
+    ap.add_argument("--offsets", type=int, nargs="+", default=[0, 256])
+    ap.add_argument("--out", required=True)
+    args = ap.parse_args(argv)
+    if not torch.cuda.is_available():
+        sys.exit("tune_weave needs the GPU it tunes for")
+    table = tune(args.hidden, args.k, args.world_size, args.tokens, args.offsets,
+                 log=lambda m: print(m, file=sys.stderr, flush=True))
+    with open(args.out, "w") as f:
+        json.dump(table, f, indent=2)
+        f.write("\n")
+    print(args.out)
+
+
+if __name__ == "__main__":
+    main()

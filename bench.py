@@ -327,7 +327,7 @@ def main():
                            "gbps": round(c.bytes / r["kernel_us_mean"] / 1e3, 1),
                            "pct_hbm_peak": round(c.bytes / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
             log(f"[sweep] {name}: {sweep[name]}")
-        w = time_weave(device, norm_cap=0, gemm_cap=160)
+        w = time_weave(device, norm_cap=0, gemm_cap=128)
         sweep["c5_weave"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}
         log(f"[sweep] c5_weave: {sweep['c5_weave']}")
         out["sweep"] = sweep

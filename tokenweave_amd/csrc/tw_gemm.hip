@@ -10,10 +10,12 @@
 // with 4 consecutive n per accumulator quad: 8-byte row-major stores.
 //
 // Two kernels:
-//  * gemm_bf16_nt_big_kernel (K % 64 == 0): 256 x 256 x 64 tiles, 8 waves
-//    (2 x 4, two per SIMD), each wave 128 x 64 (128 fp32 accumulators).  Operand
+//  * gemm_bf16_nt_big_kernel<TM> (K % 64 == 0): (64 TM) x 256 x 64 tiles, TM = 3,
+//    4 or 5 chosen per problem so that the tile count wastes the fewest workgroup
+//    rounds (M = 2458: 320-row tiles make exactly 256 tiles), 8 waves (2 x 4, two
+//    per SIMD), each wave (32 TM) x 64 (up to 160 fp32 accumulators).  Operand
 //    slabs go from global memory straight into LDS (buffer_load ... lds: no
-//    staging registers, no LDS store instructions), two LDS stages of 64 KiB.
+//    staging registers, no LDS store instructions), two LDS stages of 56-72 KiB.
 //    A wave instruction fills 1 KiB = 8 LDS rows of 128 bytes; row r keeps its
 //    16-byte chunk c at position c ^ ((r >> 1) & 7), which makes the 16-byte
 //    fragment reads of 16 consecutive rows conflict-free on the 64-bank LDS
@@ -28,6 +30,8 @@
 // workgroups of one XCD (blockIdx % 8) share operand panels in that XCD's L2.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <atomic>
 
 #include "tw_common.h"
 
@@ -170,34 +174,60 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_nt_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// 256 x 256 x 64 tiles, direct-to-LDS operand slabs (see the file comment).
+// (32 TM x 2) x 256 x 64 tiles, direct-to-LDS operand slabs (see the file
+// comment).  TM = 32-row MFMA tiles per wave along M: 4 -> 256-row tiles,
+// 5 -> 320-row tiles, 3 -> 192-row tiles.  The launcher picks the height that
+// wastes the fewest workgroup rounds for the given M.
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void lds_void_t;
-constexpr int BIG_BM = 256, BIG_BN = 256, BIG_BK = 64;
+constexpr int BIG_BN = 256, BIG_BK = 64;
 constexpr int BIG_THREADS = 512;
 constexpr int BIG_ROWB = BIG_BK * 2;             // bytes per LDS row
-constexpr int BIG_PANEL = BIG_BM * BIG_ROWB;     // 32 KiB: one operand, one stage
-constexpr int BIG_STAGE = 2 * BIG_PANEL;         // a-panel then b-panel
-constexpr int BIG_LDS_BYTES = 2 * BIG_STAGE;     // two stages
+constexpr int BIG_PANEL_B = BIG_BN * BIG_ROWB;   // 32 KiB: the b operand, one stage
 constexpr int BIG_GROUP_M = 4;
+constexpr int big_lds_bytes(int tm) { return 2 * (tm * 64 * BIG_ROWB + BIG_PANEL_B); }
 
+// One k-slab of both operands, global memory -> LDS: this wave's LA + LB wave
+// instructions of 1 KiB each.  (A free function, not a lambda: the kernel is a
+// template, and the host pass must be able to instantiate its stub without
+// compiling device builtins.)
+template <int LA, int LB>
+__device__ __forceinline__ void big_issue_slab(__amdgpu_buffer_rsrc_t da, __amdgpu_buffer_rsrc_t db,
+                                               const uint32_t (&va)[LA], const uint32_t (&vb)[LB],
+                                               uint8_t* sa, uint8_t* sb, uint32_t koff) {
+#pragma unroll
+  for (int j = 0; j < LA; ++j)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(da, (lds_void_t*)(sa + j * 1024), 16, va[j], koff, 0, 0);
+#pragma unroll
+  for (int j = 0; j < LB; ++j)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(db, (lds_void_t*)(sb + j * 1024), 16, vb[j], koff, 0, 0);
+}
+
+template <int TM>
 __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
     int M, int N, int K, int64_t ldc, int tiles_m, int tiles_n) {
-  constexpr int TM = 4, TN = 2;  // 32 x 32 MFMA tiles per wave: 128 x 64
+  constexpr int TN = 2;                 // wave tile (32 TM) x 64
+  constexpr int WM = 32 * TM;           // rows per wave
+  constexpr int BM = 2 * WM;            // rows per workgroup tile
+  constexpr int PANEL_A = BM * BIG_ROWB;
+  constexpr int STAGE = PANEL_A + BIG_PANEL_B;  // a-panel then b-panel
+  constexpr int LA = BM / 64;           // a-panel loads per wave per slab (8 rows x 8 waves each)
+  constexpr int LB = BIG_BN / 64;       // b-panel loads per wave per slab
+  constexpr int H1 = (TM + 1) / 2;      // MFMA rows issued before the next fragments are fetched
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds_big[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 2, wn = wave & 3, l32 = lane & 31, lhi = lane >> 5;
   const int num_tiles = tiles_m * tiles_n;
   const int nk = K / BIG_BK;
-  // Loader: wave instruction j of wave w fills LDS rows [(4w + j) * 8, +8); lane l
-  // lands at row l / 8, position l % 8, so it must fetch chunk (l % 8) ^ key(row).
+  // Loader: wave instruction j of wave w fills the 8-row LDS block w * L + j; lane l
+  // lands at row l / 8, position l % 8 of that block, so it must fetch the chunk
+  // (l % 8) ^ key(row), key(r) = (r >> 1) & 7 = ((block & 1) << 2) | (l >> 4).
   const int ld_row = lane >> 3;
-  const int ld_key = lane >> 4;                     // key of rows in an even 8-row block
-  const int ld_chunk_even = (lane & 7) ^ ld_key;
-  const int ld_chunk_odd = (lane & 7) ^ (ld_key | 4);  // odd block: rows 8..15 of a 16-row group
-  // Reader: lane row l32 (+ 32 i), chunk 2 kk + lhi.
+  const int ld_key = lane >> 4;
+  // Reader: lane row l32 (+ 32 i; wave offsets are multiples of 16 rows, which do not
+  // change the key), chunk 2 kk + lhi.
   uint32_t roff[4];
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk)
@@ -221,27 +251,21 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
     const int rows_in_group = min(tiles_m - first_m, BIG_GROUP_M);
     const int tm_idx = first_m + (pid % group_size) % rows_in_group;
     const int tn_idx = (pid % group_size) / rows_in_group;
-    const int m0 = tm_idx * BIG_BM, n0 = tn_idx * BIG_BN;
+    const int m0 = tm_idx * BM, n0 = tn_idx * BIG_BN;
 
-    uint32_t va[4], vb[4];
+    uint32_t va[LA], vb[LB];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int r = (wave * 4 + j) * 8 + ld_row;
-      const int chunk = (j & 1) ? ld_chunk_odd : ld_chunk_even;  // 4 * wave is even
-      va[j] = (uint32_t)(((size_t)(m0 + r) * K + chunk * 8) * 2);
-      vb[j] = (uint32_t)(((size_t)(n0 + r) * K + chunk * 8) * 2);
+    for (int j = 0; j < LA; ++j) {
+      const int blk = wave * LA + j;
+      const int chunk = (lane & 7) ^ (((blk & 1) << 2) | ld_key);
+      va[j] = (uint32_t)(((size_t)(m0 + blk * 8 + ld_row) * K + chunk * 8) * 2);
     }
-    auto issue = [&](int kt, int stage) {
-      uint8_t* sa = lds_big + stage * BIG_STAGE + (wave * 4) * 1024;
-      uint8_t* sb = sa + BIG_PANEL;
-      const uint32_t koff = (uint32_t)kt * BIG_ROWB;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(da, (lds_void_t*)(sa + j * 1024), 16, va[j], koff, 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(db, (lds_void_t*)(sb + j * 1024), 16, vb[j], koff, 0, 0);
-      }
-    };
-
+    for (int j = 0; j < LB; ++j) {
+      const int blk = wave * LB + j;
+      const int chunk = (lane & 7) ^ (((blk & 1) << 2) | ld_key);
+      vb[j] = (uint32_t)(((size_t)(n0 + blk * 8 + ld_row) * K + chunk * 8) * 2);
+    }
     f32x16_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -251,15 +275,19 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
     __syncthreads();  // the previous tile's fragment reads are finished
-    issue(0, 0);
+    big_issue_slab<LA, LB>(da, db, va, vb, lds_big + (wave * LA) * 1024,
+                           lds_big + PANEL_A + (wave * LB) * 1024, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     for (int kt = 0; kt < nk; ++kt) {
       const int stage = kt & 1;
-      if (kt + 1 < nk) issue(kt + 1, stage ^ 1);
-      const uint8_t* pa = lds_big + stage * BIG_STAGE + (wm * 128) * BIG_ROWB;
-      const uint8_t* pb = lds_big + stage * BIG_STAGE + BIG_PANEL + (wn * 64) * BIG_ROWB;
+      if (kt + 1 < nk)
+        big_issue_slab<LA, LB>(da, db, va, vb, lds_big + (stage ^ 1) * STAGE + (wave * LA) * 1024,
+                               lds_big + (stage ^ 1) * STAGE + PANEL_A + (wave * LB) * 1024,
+                               (uint32_t)(kt + 1) * BIG_ROWB);
+      const uint8_t* pa = lds_big + stage * STAGE + (wm * WM) * BIG_ROWB;
+      const uint8_t* pb = lds_big + stage * STAGE + PANEL_A + (wn * 64) * BIG_ROWB;
       bf16x8_t fa[2][TM], fb[2][TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -270,12 +298,12 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
         const int cur = kk & 1, nxt = cur ^ 1;
-        // First half of this step's MFMAs, the next step's fragment reads, second
-        // half: the reads complete in the shadow of the second half.  The
-        // scheduling barriers keep the compiler from sinking the reads to their use.
+        // First part of this step's MFMAs, the next step's fragment reads, the rest:
+        // the reads complete in the shadow of the rest.  The scheduling barriers keep
+        // the compiler from sinking the reads to their use.
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < TM / 2; ++i)
+        for (int i = 0; i < H1; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
@@ -292,7 +320,7 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = TM / 2; i < TM; ++i)
+        for (int i = H1; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
@@ -304,10 +332,10 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
       __syncthreads();
     }
 
-    // acc[i][j][4 q + e] = out[m0 + wm*128 + i*32 + l32][n0 + wn*64 + j*32 + 8 q + 4 lhi + e]
+    // acc[i][j][4 q + e] = out[m0 + wm*WM + i*32 + l32][n0 + wn*64 + j*32 + 8 q + 4 lhi + e]
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int m = m0 + wm * 128 + i * 32 + l32;
+      const int m = m0 + wm * WM + i * 32 + l32;
       if (m >= M) continue;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
@@ -324,6 +352,45 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
       }
     }
   }
+}
+
+
+template <int TM>
+static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64_t M, int64_t N,
+                      int64_t K, int64_t ldc, int max_cus, hipStream_t hs) {
+  constexpr int BM = 64 * TM;
+  constexpr int LDS = big_lds_bytes(TM);
+  static std::atomic<bool> lds_ok{false};
+  if (!lds_ok.load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_big_kernel<TM>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess)
+      return set_error(TW_ERR_LAUNCH, "gemm_bf16_nt: the device refused %d bytes of LDS", LDS);
+    lds_ok.store(true, std::memory_order_release);
+  }
+  const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BIG_BN - 1) / BIG_BN);
+  int64_t grid = (int64_t)tiles_m * tiles_n;
+  if (max_cus > 0 && grid > max_cus) grid = max_cus;
+  hipLaunchKernelGGL(gemm_bf16_nt_big_kernel<TM>, dim3((unsigned)grid), dim3(BIG_THREADS), LDS, hs, out, a,
+                     b, (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n);
+  return TW_OK;
+}
+
+// Tile height (in 64-row units) that finishes soonest on `cus` compute units: time is
+// proportional to rounds x tile height; ties go to the smaller tile.
+static int pick_tile_height(int64_t M, int64_t N, int cus) {
+  const int64_t tiles_n = (N + BIG_BN - 1) / BIG_BN;
+  int best = 4;
+  int64_t best_cost = INT64_MAX;
+  for (int tm : {3, 4, 5}) {
+    const int64_t tiles = ((M + 64 * tm - 1) / (64 * tm)) * tiles_n;
+    const int64_t rounds = (tiles + cus - 1) / cus;
+    const int64_t cost = rounds * tm * 64 + 8;  // +8: per-round fixed part (prologue, epilogue)
+    if (cost < best_cost || (cost == best_cost && tm < best)) {
+      best = tm;
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t N, int64_t K,
@@ -344,19 +411,18 @@ int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t
   const bool big = (K % BIG_BK == 0) && ((uint64_t)M * K < (1ull << 31)) && ((uint64_t)N * K < (1ull << 31)) &&
                    M >= 192 && N >= 192;
   if (big) {
-    static bool lds_ok = false;  // benign race: the attribute call is idempotent
-    if (!lds_ok) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_big_kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, BIG_LDS_BYTES) != hipSuccess)
-        return set_error(TW_ERR_LAUNCH, "gemm_bf16_nt: the device refused %d bytes of LDS", BIG_LDS_BYTES);
-      lds_ok = true;
+    int cus = max_cus > 0 ? max_cus : device_compute_units();
+    if (cus <= 0) cus = 256;
+    uint16_t* o = static_cast<uint16_t*>(out);
+    const uint16_t* pa = static_cast<const uint16_t*>(a);
+    const uint16_t* pb = static_cast<const uint16_t*>(b);
+    int rc;
+    switch (pick_tile_height(M, N, cus)) {
+      case 3: rc = launch_big<3>(o, pa, pb, M, N, K, ldc, max_cus, hs); break;
+      case 5: rc = launch_big<5>(o, pa, pb, M, N, K, ldc, max_cus, hs); break;
+      default: rc = launch_big<4>(o, pa, pb, M, N, K, ldc, max_cus, hs); break;
     }
-    const int tiles_m = (int)((M + BIG_BM - 1) / BIG_BM), tiles_n = (int)((N + BIG_BN - 1) / BIG_BN);
-    int64_t grid = (int64_t)tiles_m * tiles_n;
-    if (max_cus > 0 && grid > max_cus) grid = max_cus;
-    hipLaunchKernelGGL(gemm_bf16_nt_big_kernel, dim3((unsigned)grid), dim3(BIG_THREADS), BIG_LDS_BYTES, hs,
-                       static_cast<uint16_t*>(out), static_cast<const uint16_t*>(a),
-                       static_cast<const uint16_t*>(b), (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n);
+    if (rc != TW_OK) return rc;
   } else {
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
     int64_t grid = (int64_t)tiles_m * tiles_n;

@@ -280,6 +280,29 @@ def test_runs_on_the_current_torch_stream(oracle):
     assert np.array_equal(to_bits(out), y0) and np.array_equal(to_bits(res), r0)
 
 
+def test_rows_beyond_4_gib_are_addressed_with_64_bit_offsets(oracle):
+    """270 000 rows x 8192 = 4.4 GB per tensor: row offsets do not fit 32 bits.  Rows are
+    independent, so a sample of rows is checked against the checker run on those rows."""
+    T, H = 270_000, 8192
+    g = torch.Generator(device=DEV)
+    g.manual_seed(99)
+    x = torch.empty(T, H, dtype=torch.bfloat16, device=DEV)
+    r = torch.empty(T, H, dtype=torch.bfloat16, device=DEV)
+    for lo in range(0, T, 30_000):   # fill in slabs to bound the fp32 temporaries
+        hi = min(T, lo + 30_000)
+        x[lo:hi] = torch.randn(hi - lo, H, generator=g, device=DEV)
+        r[lo:hi] = torch.randn(hi - lo, H, generator=g, device=DEV)
+    w = (1 + 0.1 * torch.randn(H, generator=g, device=DEV)).to(torch.bfloat16)
+    rows = torch.tensor([0, 1, 131_071, 131_072, 262_143, 262_144, T - 2, T - 1], device=DEV)
+    x_s, r_s = to_bits(x[rows]), to_bits(r[rows])
+    oracle.fused_add_rms_norm(x_s, r_s, to_bits(w), 1e-5)
+    ops.fused_add_rms_norm(x, r, w, 1e-5)
+    torch.cuda.synchronize()
+    assert_parity(to_bits(x[rows]), to_bits(r[rows]), x_s, r_s, "rows past 4 GiB", max_y_mismatch=5e-3)
+    del x, r
+    torch.cuda.empty_cache()
+
+
 def test_op_is_capturable_in_a_hip_graph_and_replays_exactly():
     """The entry points only enqueue (no allocation, no host sync), so a caller may
     capture them.  Every replay is checked against the eager result, with eager work

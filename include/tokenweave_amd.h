@@ -46,6 +46,10 @@ extern "C" {
 #define TW_DTYPE_F16 1
 #define TW_DTYPE_F32 2
 
+/* Output kinds of the dynamic per-token quantisation ops. */
+#define TW_QUANT_FP8_E4M3FN 0
+#define TW_QUANT_INT8 1
+
 #define TW_MAX_PARTIALS 16
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -173,6 +177,34 @@ TW_API int tw_reduce_add_rms_norm_static_fp8_quant(const void* const* partials, 
                                                    const float* scale, int64_t num_tokens,
                                                    int64_t hidden_size, int max_ctas,
                                                    float epsilon, void* stream);
+
+/* Residual-add (optional) + RMSNorm + dynamic per-token quantisation:
+ *   x = input + residual (fp32) ; residual <- x ; rms = 1/sqrt(mean(x^2) + epsilon)
+ *   n = round(round(x * rms) * weight)            (both roundings to the input type)
+ *   scales[t] = max(min(max_j |n[t][j]|, *scale_ub) / qmax, floor)
+ *   out = fp8_e4m3fn(clamp(n / scales[t], +-448))     qmax 448, floor 1/(448 * 512)
+ *       | int8(saturate(rint(n * (1 / scales[t]))))   qmax 127, floor FLT_EPSILON
+ * out: [num_tokens, hidden_size] bytes; scales: num_tokens floats (device);
+ * scale_ub: NULL or one device float (fp8 only); residual: NULL or
+ * [num_tokens, hidden_size], updated in place.  input is not modified.  Any
+ * hidden_size / alignment (vector kernel for bf16, 16-byte aligned, hidden_size % 16 == 0).
+ * Replaces ::rms_norm_dynamic_per_token_quant
+ * (csrc/quantization/fused_kernels/fused_layernorm_dynamic_per_token_quant.cu:131-155,
+ * schema at csrc/torch_bindings.cpp:216-221). */
+TW_API int tw_rms_norm_dynamic_per_token_quant(void* out, const void* input, const void* weight,
+                                               float* scales, const float* scale_ub,
+                                               void* residual, int64_t num_tokens,
+                                               int64_t hidden_size, float epsilon, int dtype,
+                                               int out_kind, void* stream);
+
+/* The op above over P partial buffers: x = sum_p partials[p] + residual in fp32,
+ * fixed order.  bf16 in; 16-byte alignment and hidden_size % 16 == 0 required;
+ * residual may be NULL.  No counterpart in the reference (its TokenWeave kernels
+ * emit bf16); it fuses the reference's all-reduce + the op above. */
+TW_API int tw_reduce_add_rms_norm_dynamic_per_token_quant(
+    const void* const* partials, int num_partials, void* out, float* scales, void* residual,
+    const void* weight, const float* scale_ub, int64_t num_tokens, int64_t hidden_size,
+    int max_ctas, float epsilon, int out_kind, void* stream);
 
 /* dst[0, nbytes) <- src[0, nbytes) with a plain grid-stride copy kernel (default
  * cache policy, 16 bytes per lane).  nbytes % 16 == 0, 16-byte aligned pointers,

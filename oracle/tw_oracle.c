@@ -23,7 +23,10 @@
  * layernorm.cpp compiled from its sources (oracle/_ref, truncating build) on the
  * reference's test grid; closed forms (constant / one-hot / zero rows); an
  * independent numpy fp32 restatement of RMSNorm.forward_native; float64 witness;
- * the fp8 conversion against torch's own CPU cast over every bf16 bit pattern.
+ * the fp8 conversion against torch's own CPU cast over every bf16 bit pattern;
+ * the dynamic per-token quantisation against the composition the reference's own
+ * test uses (tests/kernels/test_fused_quant_layernorm.py:51-72): forward_native
+ * in numpy, then per-token scales and torch's CPU fp8 cast / numpy rint.
  *
  * Every function is built with -ffp-contract=off: the reference's vector code is
  * separate multiplies and adds (no FMA in its AVX2 build).
@@ -171,6 +174,78 @@ int tw_oracle_static_fp8_quant(uint8_t* out, const uint16_t* y, int64_t n, float
     float x = bf16_to_f32(y[i]) * inv;
     x = fmaxf(-448.0f, fminf(x, 448.0f));
     out[i] = f32_to_e4m3fn(x);
+  }
+  return 0;
+}
+
+/* Residual-add + RMSNorm + dynamic per-token quantisation, P partials.
+ * Follows the reference's fused kernel, scalar path
+ * (csrc/quantization/fused_kernels/layernorm_utils.cuh:19-126, called from
+ * fused_layernorm_dynamic_per_token_quant.cu:64-83); the reference has no CPU twin.
+ *   x      = sum_p f32(partial_p) + f32(r)                    (fp32; :28-31)
+ *   rms    = 1/sqrt(sum x^2 / H + eps)   (unrounded x; :34,43 uses rsqrtf, whose CUDA
+ *            implementation is within 2 ulp of this correctly rounded value)
+ *   n      = f32( bf16( f32(bf16(x * rms)) * f32(w) ) )       (two roundings; :68,114)
+ *   scale  = max( min(max_j |n_j|, *scale_ub) / qmax, min_scale )   (:80-88)
+ *            qmax = 448, min_scale = 1/(448*512) for fp8 (csrc/quantization/utils.cuh:48-52);
+ *            qmax = 127, min_scale = FLT_EPSILON for int8 (:55-59)
+ *   r      <- bf16(x)                                         (:111)
+ *   out    = fp8_rne(clamp(n / scale, +-448))   (division: quant_conversions.cuh:34-39,62-69)
+ *          | int8_sat(rint(n * (1/scale)))      (fused_layernorm_..._quant.cu:32-36,
+ *                                                quant_conversions.cuh:14-32,47-52)
+ * The sum of squares is accumulated as in row_reduce_add_norm (the reference's GPU
+ * order is a cub block reduction of unspecified association).
+ * qkind: 0 = fp8 e4m3fn, 1 = int8.  r and scale_ub may be NULL. */
+int tw_oracle_rms_norm_dynamic_per_token_quant(
+    uint8_t* out, float* scales, const uint16_t* const* partials, int P, uint16_t* r,
+    const uint16_t* w, const float* scale_ub, int64_t T, int64_t H, float eps, int qkind) {
+  if (H <= 0 || T < 0 || P < 1 || P > 64 || (qkind != 0 && qkind != 1)) return -1;
+  const float qmax = qkind == 0 ? 448.0f : 127.0f;
+  const float min_scale = qkind == 0 ? 1.0f / (448.0f * 512.0f) : 1.1920928955078125e-07f;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < T; ++i) {
+    const int64_t off = i * H;
+    float lane[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int64_t j = 0; j < H; ++j) {
+      float x = bf16_to_f32(partials[0][off + j]);
+      for (int p = 1; p < P; ++p) x = x + bf16_to_f32(partials[p][off + j]);
+      if (r) x = x + bf16_to_f32(r[off + j]);
+      float sq = x * x;
+      lane[j & 7] = lane[j & 7] + sq;
+    }
+    float ss = 0.0f;
+    for (int k = 0; k < 8; ++k) ss += lane[k];
+    const float rms = 1.0f / sqrtf(ss / (float)H + eps);
+    float amax = 0.0f;
+    for (int pass = 0; pass < 2; ++pass) {
+      float scale = 0.0f, scale_inv = 0.0f;
+      if (pass == 1) {
+        scale = scale_ub ? fminf(amax, *scale_ub) : amax;
+        scale = fmaxf(scale / qmax, min_scale);
+        scales[i] = scale;
+        scale_inv = 1.0f / scale;
+      }
+      for (int64_t j = 0; j < H; ++j) {
+        float x = bf16_to_f32(partials[0][off + j]);
+        for (int p = 1; p < P; ++p) x = x + bf16_to_f32(partials[p][off + j]);
+        if (r) x = x + bf16_to_f32(r[off + j]);
+        float t = bf16_to_f32(f32_to_bf16(x * rms, TW_ROUND_RNE));
+        float n = bf16_to_f32(f32_to_bf16(t * bf16_to_f32(w[j]), TW_ROUND_RNE));
+        if (pass == 0) {
+          amax = fmaxf(amax, fabsf(n));
+        } else {
+          if (r) r[off + j] = f32_to_bf16(x, TW_ROUND_RNE);
+          if (qkind == 0) {
+            float q = fmaxf(-448.0f, fminf(n / scale, 448.0f));
+            out[off + j] = f32_to_e4m3fn(q);
+          } else {
+            float q = rintf(n * scale_inv);
+            q = fmaxf(-128.0f, fminf(q, 127.0f));
+            out[off + j] = (uint8_t)(int8_t)q;
+          }
+        }
+      }
+    }
   }
   return 0;
 }

@@ -59,6 +59,10 @@ def lib() -> ctypes.CDLL:
         L.tw_oracle_gemm_bf16_nt.argtypes = [_u16p, _u16p, _u16p, i64, i64, i64, ci]
         L.tw_oracle_static_fp8_quant.argtypes = [ctypes.POINTER(ctypes.c_uint8), _u16p, i64, f32]
         L.tw_oracle_static_fp8_quant.restype = ci
+        L.tw_oracle_rms_norm_dynamic_per_token_quant.argtypes = [
+            ctypes.POINTER(ctypes.c_uint8), ctypes.POINTER(ctypes.c_float), ctypes.POINTER(_u16p), ci,
+            _u16p, _u16p, ctypes.POINTER(ctypes.c_float), i64, i64, f32, ci]
+        L.tw_oracle_rms_norm_dynamic_per_token_quant.restype = ci
         for name in ("fused_add_rms_norm", "reduce_add_rms_norm", "rms_norm",
                      "rms_norm_inplace", "gemm_bf16_nt"):
             getattr(L, "tw_oracle_" + name).restype = ci
@@ -156,6 +160,31 @@ def static_fp8_quant(y, scale):
     _check(lib().tw_oracle_static_fp8_quant(out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)),
                                             _p(y), y.size, scale), "static_fp8_quant")
     return out
+
+
+QUANT_FP8 = 0
+QUANT_INT8 = 1
+
+
+def rms_norm_dynamic_per_token_quant(partials, w, eps, qkind, scale_ub=None, r=None):
+    """Fused (P-partial) add + RMSNorm + dynamic per-token quantisation.
+
+    partials: list of [T, H] bf16 bit patterns; r (optional) is updated in place.
+    Returns (codes uint8 [T, H] — e4m3fn bytes or int8 two's complement, scales f32 [T, 1])."""
+    P = len(partials)
+    T, H = _th(partials[0])
+    out = np.empty(partials[0].shape, np.uint8)
+    scales = np.empty((T, 1), np.float32)
+    arr = (_u16p * P)(*[_p(a) for a in partials])
+    ub = None
+    if scale_ub is not None:
+        ub = ctypes.pointer(ctypes.c_float(float(scale_ub)))
+    _check(lib().tw_oracle_rms_norm_dynamic_per_token_quant(
+        out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)),
+        scales.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), arr, P,
+        _p(r) if r is not None else None, _p(w), ub, T, H, eps, qkind),
+        "rms_norm_dynamic_per_token_quant")
+    return out, scales
 
 
 # ----------------------------------------------------------------------------

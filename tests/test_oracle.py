@@ -314,3 +314,159 @@ def test_fp8_quant_matches_torch_cast_on_every_bf16_pattern(oracle):
     f = np.array([448.0, 1000.0, -1000.0, 0.0, 2 ** -9, 2 ** -10, 3 * 2 ** -10, 17.0, 19.0], np.float32)
     got = oracle.static_fp8_quant(oracle.f32_to_bf16(f), 1.0)
     assert list(got) == [0x7E, 0x7E, 0xFE, 0x00, 0x01, 0x00, 0x02, 0x58, 0x5A]
+
+
+# ---------------------------------------------------------------------------
+# dynamic per-token quantisation: pinned by the composition the reference's own
+# test compares its fused kernel with (tests/kernels/test_fused_quant_layernorm.py
+# :51-72): forward_native, then per-token scales, then the element conversion — here
+# in numpy, with torch's CPU cast as the fp8 converter.
+# ---------------------------------------------------------------------------
+FP8_MAX, FP8_MIN_SCALE = np.float32(448.0), np.float32(1.0 / (448.0 * 512.0))
+I8_MAX, I8_MIN_SCALE = np.float32(127.0), np.float32(np.finfo(np.float32).eps)
+
+
+def _composed_dynamic_quant(oracle, x_f32_exact_bits, r, w, eps, qkind, ub):
+    """x_f32_exact_bits: bf16 bits of the (already summed) input; returns codes, scales, r'."""
+    import torch
+    res = oracle.forward_native_np(x_f32_exact_bits, r, w, eps)
+    y, r_new = res if r is not None else (res, None)
+    n = bits_to_f32(y)
+    amax = np.abs(n).max(axis=-1, keepdims=True).astype(np.float32)
+    if qkind == oracle.QUANT_FP8:
+        s = amax if ub is None else np.minimum(amax, np.float32(ub))
+        scales = np.maximum(s / FP8_MAX, FP8_MIN_SCALE).astype(np.float32)
+        q = np.clip(n / scales, -FP8_MAX, FP8_MAX).astype(np.float32)
+        codes = torch.from_numpy(q).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    else:
+        scales = np.maximum(amax / I8_MAX, I8_MIN_SCALE).astype(np.float32)
+        q = np.rint(n * (np.float32(1.0) / scales)).astype(np.float32)
+        codes = np.clip(q, -128, 127).astype(np.int8).view(np.uint8)
+    return codes, scales, r_new
+
+
+def _order_free_bits(rng, shape, kmax=64):
+    """bf16 values k/64, |k| <= kmax: squares and their sums over <= 4096 elements are
+    exact in fp32 in any order, so every implementation agrees on the mean bit for bit."""
+    from oracle import tw_oracle as O
+    k = rng.integers(-kmax, kmax + 1, size=shape)
+    return O.f32_to_bf16((k / 64.0).astype(np.float32))
+
+
+@pytest.mark.parametrize("qkind", [0, 1])
+@pytest.mark.parametrize("add_residual", [False, True])
+@pytest.mark.parametrize("use_ub", [False, True])
+@pytest.mark.parametrize("T,H", [(1, 64), (7, 1024), (83, 2048), (5, 4096), (3, 1032)])
+def test_dynamic_quant_equals_reference_test_composition_bitwise(oracle, qkind, add_residual, use_ub, T, H):
+    if use_ub and qkind == oracle.QUANT_INT8:
+        pytest.skip("scale_ub is fp8-only (fused_layernorm_dynamic_per_token_quant.cu:144-146)")
+    rng = np.random.default_rng(100 * T + H + 7 * qkind)
+    x = _order_free_bits(rng, (T, H), kmax=32)
+    r = _order_free_bits(rng, (T, H), kmax=32) if add_residual else None
+    w = oracle.f32_to_bf16(rng.normal(1.0, 0.1, H).astype(np.float32))
+    eps = 1e-6
+    ub = None
+    if use_ub:
+        # as in the reference test (:139-141): the mean of the normalised output
+        yy = oracle.forward_native_np(x, r, w, eps)
+        yy = yy[0] if add_residual else yy
+        ub = float(np.abs(bits_to_f32(yy)).mean())
+    want_codes, want_scales, want_r = _composed_dynamic_quant(oracle, x, r, w, eps, qkind, ub)
+    r_io = r.copy() if add_residual else None
+    codes, scales = oracle.rms_norm_dynamic_per_token_quant([x], w, eps, qkind, scale_ub=ub, r=r_io)
+    assert np.array_equal(scales, want_scales)
+    assert np.array_equal(codes, want_codes), int((codes != want_codes).sum())
+    if add_residual:
+        assert np.array_equal(r_io, want_r)
+    if use_ub:
+        assert (np.abs(bits_to_f32(yy)).max(axis=-1) > ub).any(), "the bound never bites: test is vacuous"
+
+
+@pytest.mark.parametrize("qkind", [0, 1])
+def test_dynamic_quant_partials_sum_in_fp32_before_anything_is_rounded(oracle, qkind):
+    """P order-free partials == one input holding their exact sum."""
+    rng = np.random.default_rng(5)
+    T, H, P = 6, 2048, 8
+    parts = [_order_free_bits(rng, (T, H), kmax=4) for _ in range(P)]
+    total = oracle.f32_to_bf16(sum(bits_to_f32(p) for p in parts))   # |k| <= 32: exact in bf16
+    r = _order_free_bits(rng, (T, H), kmax=32)
+    w = oracle.f32_to_bf16(rng.normal(1.0, 0.1, H).astype(np.float32))
+    r1, r2 = r.copy(), r.copy()
+    c1, s1 = oracle.rms_norm_dynamic_per_token_quant(parts, w, 1e-6, qkind, r=r1)
+    c2, s2 = oracle.rms_norm_dynamic_per_token_quant([total], w, 1e-6, qkind, r=r2)
+    assert np.array_equal(c1, c2) and np.array_equal(s1, s2) and np.array_equal(r1, r2)
+
+
+@pytest.mark.parametrize("T,H", [(7, 768), (83, 5120), (16, 8192)])
+@pytest.mark.parametrize("qkind", [0, 1])
+def test_dynamic_quant_random_rows_within_reference_test_tolerance(oracle, qkind, T, H):
+    """Random data (the reference test's distribution): the mean of squares may differ
+    from numpy's pairwise mean in the last bit, which can move a rounding; the reference's
+    test allows rtol 1e-5 on scales and one step on int8 codes
+    (test_fused_quant_layernorm.py:151-159).  Here: almost every row exact, none off by
+    more than one bf16 step of the row maximum."""
+    rng = np.random.default_rng(11 * T + H)
+    x = rand_bits(rng, (T, H), 1.0 / H)
+    r = rand_bits(rng, (T, H), 1.0 / H)
+    w = oracle.f32_to_bf16(rng.normal(1.0, 0.1, H).astype(np.float32))
+    want_codes, want_scales, want_r = _composed_dynamic_quant(oracle, x, r, w, 1e-6, qkind, None)
+    r_io = r.copy()
+    codes, scales = oracle.rms_norm_dynamic_per_token_quant([x], w, 1e-6, qkind, r=r_io)
+    assert np.array_equal(r_io, want_r)
+    rel = np.abs(scales - want_scales) / want_scales
+    assert rel.max() <= 2.0 ** -7 and (rel > 1e-5).mean() <= 0.05
+    same_scale = (rel[:, 0] == 0)
+    a = codes[same_scale].view(np.int8).astype(np.int32)
+    b = want_codes[same_scale].view(np.int8).astype(np.int32)
+    if qkind == oracle.QUANT_FP8:   # sign-magnitude codes -> monotone line
+        a = np.where(a < 0, -(a & 0x7F), a)
+        b = np.where(b < 0, -(b & 0x7F), b)
+    d = np.abs(a - b)
+    assert d.max() <= 1 and (d != 0).mean() <= 2e-3
+
+
+def test_dynamic_quant_closed_forms(oracle):
+    H = 512
+    w1 = oracle.f32_to_bf16(np.ones(H, np.float32))
+    # constant row: every element is the row maximum -> every code is the largest one
+    x = oracle.f32_to_bf16(np.full((1, H), -0.75, np.float32))
+    c, s = oracle.rms_norm_dynamic_per_token_quant([x], w1, 1e-6, oracle.QUANT_FP8)
+    assert (c == 0xFE).all()                      # -448
+    assert abs(s[0, 0] * 448.0 - 1.0) < 2.0 ** -8  # |n| = bf16(0.75 / sqrt(0.5625 + eps)) ~ 1
+    c, s = oracle.rms_norm_dynamic_per_token_quant([x], w1, 1e-6, oracle.QUANT_INT8)
+    assert (c.view(np.int8) == -127).all() and abs(s[0, 0] * 127.0 - 1.0) < 2.0 ** -8
+    # one-hot row: n_k = a / sqrt(a^2 / H) = sqrt(H) up to the eps term, scale = n_k / qmax
+    x = np.zeros((1, H), np.float32); x[0, 5] = 3.0
+    c, s = oracle.rms_norm_dynamic_per_token_quant([oracle.f32_to_bf16(x)], w1, 1e-6, oracle.QUANT_FP8)
+    assert c[0, 5] == 0x7E and (np.delete(c[0], 5) == 0).all()
+    assert abs(s[0, 0] * 448.0 / np.sqrt(H) - 1.0) < 2.0 ** -7
+    # zero row: the scale floor, zero codes
+    z = np.zeros((2, H), np.uint16)
+    c, s = oracle.rms_norm_dynamic_per_token_quant([z], w1, 1e-6, oracle.QUANT_FP8)
+    assert (c == 0).all() and (s == FP8_MIN_SCALE).all()
+    c, s = oracle.rms_norm_dynamic_per_token_quant([z], w1, 1e-6, oracle.QUANT_INT8)
+    assert (c == 0).all() and (s == I8_MIN_SCALE).all()
+    # upper bound below the maximum: scale = ub / 448 and everything above ub saturates
+    rng = np.random.default_rng(3)
+    x = rand_bits(rng, (4, H))
+    c, s = oracle.rms_norm_dynamic_per_token_quant([x], w1, 1e-6, oracle.QUANT_FP8, scale_ub=0.5)
+    assert np.array_equal(s, np.full((4, 1), np.float32(0.5) / FP8_MAX, np.float32))
+    n = bits_to_f32(oracle.forward_native_np(x, None, w1, 1e-6))
+    assert ((c & 0x7F) == 0x7E)[np.abs(n) >= 0.5].all() and (np.abs(n) >= 0.5).any()
+
+
+def test_dynamic_quant_dequantises_to_the_normalised_output(oracle):
+    """codes * scale reproduces forward_native's output to the format's precision:
+    fp8 e4m3 relative 2^-4 (plus its subnormal step), int8 half a step."""
+    import torch
+    rng = np.random.default_rng(17)
+    T, H = 9, 4096
+    x, r = rand_bits(rng, (T, H)), rand_bits(rng, (T, H))
+    w = oracle.f32_to_bf16(rng.uniform(0.5, 1.5, H).astype(np.float32))
+    n = bits_to_f32(oracle.forward_native_np(x, r, w, 1e-5)[0]).astype(np.float64)
+    c, s = oracle.rms_norm_dynamic_per_token_quant([x], w, 1e-5, oracle.QUANT_FP8, r=r.copy())
+    deq = torch.from_numpy(c.copy()).view(torch.float8_e4m3fn).float().numpy().astype(np.float64) * s
+    assert (np.abs(deq - n) <= np.abs(n) * 2.0 ** -4 + s * 2.0 ** -10 + 1e-2 * np.abs(n)).all()
+    c, s = oracle.rms_norm_dynamic_per_token_quant([x], w, 1e-5, oracle.QUANT_INT8, r=r.copy())
+    deq = c.view(np.int8).astype(np.float64) * s
+    assert (np.abs(deq - n) <= 0.5 * s * (1 + 1e-6) + 1e-2 * np.abs(n)).all()

@@ -339,6 +339,95 @@ def reduce_add_rms_norm_static_fp8_quant(partials: Sequence[torch.Tensor], resul
             _cap(MAX_CTAS), epsilon, _stream_ptr(residual)))
 
 
+# ---------------------------------------------------------------------------
+# norm + dynamic per-token quantisation (vllm/_custom_ops.py:256-272 ->
+# csrc/quantization/fused_kernels/fused_layernorm_dynamic_per_token_quant.cu)
+# ---------------------------------------------------------------------------
+QUANT_FP8_E4M3FN, QUANT_INT8 = 0, 1
+
+
+def _check_dyn_quant(result, like, scales, scale_ub, T):
+    """The launcher's checks (fused_layernorm_dynamic_per_token_quant.cu:139-147)."""
+    _require(result.is_cuda and result.device == like.device,
+             f"result is on {result.device}, expected {like.device}")
+    _require(result.dtype in (FP8_DTYPE, torch.int8),
+             f"result must be {FP8_DTYPE} or torch.int8, got {result.dtype}")
+    _require(result.is_contiguous() and result.shape == like.shape,
+             "result must be contiguous and have the input's shape")
+    _require(scales.is_cuda and scales.device == like.device and scales.dtype == torch.float32,
+             "scales must be a float32 tensor on the input's device")
+    _require(scales.is_contiguous() and scales.numel() == T, f"scales must hold {T} contiguous values")
+    if scale_ub is not None:
+        _require(result.dtype == FP8_DTYPE, "scale_ub is defined for fp8 output only")
+        _check_scale(scale_ub, like.device)
+    return QUANT_FP8_E4M3FN if result.dtype == FP8_DTYPE else QUANT_INT8
+
+
+def rms_norm_dynamic_per_token_quant_out(result: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,
+                                         scale: torch.Tensor, epsilon: float,
+                                         scale_ub: Optional[torch.Tensor] = None,
+                                         residual: Optional[torch.Tensor] = None) -> None:
+    """The registered op (schema csrc/torch_bindings.cpp:216-219): result, scale and
+    residual are written in place."""
+    code = _dtype_code("rms_norm_dynamic_per_token_quant_dispatch", input)
+    _check_tensor("input", input, input.dtype, input.device)
+    T, H = _rows(input)
+    kind = _check_dyn_quant(result, input, scale, scale_ub, T)
+    _check_weight(weight, H, input.dtype, input.device)
+    if residual is not None:
+        _check_tensor("residual", residual, input.dtype, input.device)
+        _require(residual.shape == input.shape, "input and residual must have the same shape")
+    with _on_device(input):
+        _lib.check(_lib.lib().tw_rms_norm_dynamic_per_token_quant(
+            result.data_ptr(), input.data_ptr(), weight.data_ptr(), scale.data_ptr(),
+            scale_ub.data_ptr() if scale_ub is not None else None,
+            residual.data_ptr() if residual is not None else None, T, H, epsilon, code, kind,
+            _stream_ptr(input)))
+
+
+def rms_norm_dynamic_per_token_quant(input: torch.Tensor, weight: torch.Tensor, epsilon: float,
+                                     quant_dtype: torch.dtype,
+                                     scale_ub: Optional[torch.Tensor] = None,
+                                     residual: Optional[torch.Tensor] = None):
+    """vllm/_custom_ops.py:256-272: allocates the outputs, returns (output, scales);
+    residual (if given) is updated in place."""
+    output = torch.empty_like(input, dtype=quant_dtype)
+    scales = torch.empty((input.numel() // input.shape[-1], 1), device=input.device, dtype=torch.float32)
+    rms_norm_dynamic_per_token_quant_out(output, input, weight, scales, epsilon, scale_ub, residual)
+    return output, scales
+
+
+def reduce_add_rms_norm_dynamic_per_token_quant(partials: Sequence[torch.Tensor], result: torch.Tensor,
+                                                scales: torch.Tensor, residual: Optional[torch.Tensor],
+                                                weight: torch.Tensor, epsilon: float,
+                                                scale_ub: Optional[torch.Tensor] = None,
+                                                MAX_CTAS: Optional[int] = None) -> None:
+    """result <- dynamic per-token quantisation of RMSNorm(sum_p partials[p] + residual) * weight,
+    scales <- the row scales, residual <- the sum (when given)."""
+    P = len(partials)
+    _require(1 <= P <= _lib.TW_MAX_PARTIALS,
+             f"number of partials {P} not in [1, {_lib.TW_MAX_PARTIALS}]")
+    first = partials[0]
+    _require_bf16("reduce_add_rms_norm_kernel", first)
+    dev = first.device
+    T, H = _rows(first)
+    for i, p in enumerate(partials):
+        _check_tensor(f"partials[{i}]", p, torch.bfloat16, dev)
+        _require(p.shape == first.shape, f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(first.shape)}")
+    if residual is not None:
+        _check_tensor("residual", residual, torch.bfloat16, dev)
+        _require(residual.shape == first.shape, "partials and residual must have the same shape")
+    kind = _check_dyn_quant(result, first, scales, scale_ub, T)
+    _check_weight(weight, H, torch.bfloat16, dev)
+    ptrs = (ctypes.c_void_p * P)(*[p.data_ptr() for p in partials])
+    with _on_device(first):
+        _lib.check(_lib.lib().tw_reduce_add_rms_norm_dynamic_per_token_quant(
+            ptrs, P, result.data_ptr(), scales.data_ptr(),
+            residual.data_ptr() if residual is not None else None, weight.data_ptr(),
+            scale_ub.data_ptr() if scale_ub is not None else None, T, H, _cap(MAX_CTAS), epsilon, kind,
+            _stream_ptr(first)))
+
+
 def gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
                  max_cus: Optional[int] = None) -> None:
     """out[M, N] <- a[M, K] @ b[N, K]^T (bf16, fp32 accumulate).  `out` may be a row
@@ -406,6 +495,10 @@ SCHEMAS = {
     "fused_add_rms_norm_static_fp8_quant":
         "fused_add_rms_norm_static_fp8_quant(Tensor! result, Tensor input, Tensor! residual, "
         "Tensor weight, Tensor scale, float epsilon) -> ()",
+    # csrc/torch_bindings.cpp:216-219
+    "rms_norm_dynamic_per_token_quant":
+        "rms_norm_dynamic_per_token_quant(Tensor! result, Tensor input, Tensor weight, Tensor! scale, "
+        "float epsilon, Tensor? scale_ub, Tensor!? residual) -> ()",
 }
 
 _IMPLS = {
@@ -417,6 +510,7 @@ _IMPLS = {
     "fused_rs_ln_cta": fused_rs_ln_cta,
     "rms_norm_static_fp8_quant": rms_norm_static_fp8_quant,
     "fused_add_rms_norm_static_fp8_quant": fused_add_rms_norm_static_fp8_quant,
+    "rms_norm_dynamic_per_token_quant": rms_norm_dynamic_per_token_quant_out,
 }
 
 

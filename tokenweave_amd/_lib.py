@@ -43,6 +43,9 @@ PROTOTYPES = {
     "tw_fused_add_rms_norm_static_fp8_quant": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _ci, _vp],
     "tw_reduce_add_rms_norm_static_fp8_quant": [ctypes.POINTER(_vp), _ci, _vp, _vp, _vp, _vp, _i64, _i64,
                                                 _ci, _f32, _vp],
+    "tw_rms_norm_dynamic_per_token_quant": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _ci, _ci, _vp],
+    "tw_reduce_add_rms_norm_dynamic_per_token_quant": [ctypes.POINTER(_vp), _ci, _vp, _vp, _vp, _vp, _vp,
+                                                       _i64, _i64, _ci, _f32, _ci, _vp],
     "tw_copy_bytes": [_vp, _vp, _i64, _vp],
 }
 

@@ -171,6 +171,38 @@ int tw_reduce_add_rms_norm_static_fp8_quant(const void* const* partials, int num
                           TW_DTYPE_BF16, max_ctas, true, stream);
 }
 
+static int dyn_quant_kind(const char* what, int out_kind, int* quant) {
+  if (out_kind == TW_QUANT_FP8_E4M3FN) *quant = 2;
+  else if (out_kind == TW_QUANT_INT8) *quant = 3;
+  else return tw::set_error(TW_ERR_DTYPE, "%s: unknown output kind %d", what, out_kind);
+  return TW_OK;
+}
+
+int tw_rms_norm_dynamic_per_token_quant(void* out, const void* input, const void* weight,
+                                        float* scales, const float* scale_ub, void* residual,
+                                        int64_t num_tokens, int64_t hidden_size, float epsilon,
+                                        int dtype, int out_kind, void* stream) {
+  int quant;
+  if (int rc = dyn_quant_kind("rms_norm_dynamic_per_token_quant", out_kind, &quant)) return rc;
+  const void* parts[1] = {input};
+  return tw::run_row_norm_q("rms_norm_dynamic_per_token_quant", parts, 1, out, residual, nullptr,
+                            weight, quant, scale_ub, scales, num_tokens, hidden_size, epsilon, dtype,
+                            0, false, stream);
+}
+
+int tw_reduce_add_rms_norm_dynamic_per_token_quant(const void* const* partials, int num_partials,
+                                                   void* out, float* scales, void* residual,
+                                                   const void* weight, const float* scale_ub,
+                                                   int64_t num_tokens, int64_t hidden_size,
+                                                   int max_ctas, float epsilon, int out_kind,
+                                                   void* stream) {
+  int quant;
+  if (int rc = dyn_quant_kind("reduce_add_rms_norm_dynamic_per_token_quant", out_kind, &quant)) return rc;
+  return tw::run_row_norm_q("reduce_add_rms_norm_dynamic_per_token_quant", partials, num_partials, out,
+                            residual, nullptr, weight, quant, scale_ub, scales, num_tokens,
+                            hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true, stream);
+}
+
 int tw_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
   return tw::run_copy16(dst, src, nbytes, stream);
 }

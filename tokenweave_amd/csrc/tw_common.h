@@ -20,6 +20,12 @@ int run_row_norm(const char* what, const void* const* partials, int np, void* y,
                  int64_t T, int64_t H, float eps, int dtype, int max_ctas, bool require_vec,
                  void* stream);
 
+// quant: 0 none, 1 static fp8, 2 dynamic per-token fp8, 3 dynamic per-token int8.
+int run_row_norm_q(const char* what, const void* const* partials, int np, void* y,
+                   void* residual, void* copy_out, const void* weight, int quant,
+                   const float* quant_scale, float* row_scales, int64_t T, int64_t H, float eps,
+                   int dtype, int max_ctas, bool require_vec, void* stream);
+
 int run_copy16(void* dst, const void* src, int64_t nbytes, void* stream);
 
 int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t N,

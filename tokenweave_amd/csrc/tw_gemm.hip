@@ -180,12 +180,11 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_nt_kernel(
 // wastes the fewest workgroup rounds for the given M.
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void lds_void_t;
-constexpr int BIG_BN = 256, BIG_BK = 64;
+constexpr int BIG_BK = 64;
 constexpr int BIG_THREADS = 512;
 constexpr int BIG_ROWB = BIG_BK * 2;             // bytes per LDS row
-constexpr int BIG_PANEL_B = BIG_BN * BIG_ROWB;   // 32 KiB: the b operand, one stage
 constexpr int BIG_GROUP_M = 4;
-constexpr int big_lds_bytes(int tm) { return 2 * (tm * 64 * BIG_ROWB + BIG_PANEL_B); }
+constexpr int big_lds_bytes(int tm, int tn) { return 2 * (tm * 64 + tn * 128) * BIG_ROWB; }
 
 // One k-slab of both operands, global memory -> LDS: this wave's LA + LB wave
 // instructions of 1 KiB each.  (A free function, not a lambda: the kernel is a
@@ -203,17 +202,16 @@ __device__ __forceinline__ void big_issue_slab(__amdgpu_buffer_rsrc_t da, __amdg
     __builtin_amdgcn_raw_ptr_buffer_load_lds(db, (lds_void_t*)(sb + j * 1024), 16, vb[j], koff, 0, 0);
 }
 
-template <int TM>
+template <int TM, int TN>
 __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
     int M, int N, int K, int64_t ldc, int tiles_m, int tiles_n) {
-  constexpr int TN = 2;                 // wave tile (32 TM) x 64
-  constexpr int WM = 32 * TM;           // rows per wave
-  constexpr int BM = 2 * WM;            // rows per workgroup tile
+  constexpr int WM = 32 * TM, WN = 32 * TN;  // wave tile
+  constexpr int BM = 2 * WM, BN = 4 * WN;    // workgroup tile: the 8 waves as 2 x 4
   constexpr int PANEL_A = BM * BIG_ROWB;
-  constexpr int STAGE = PANEL_A + BIG_PANEL_B;  // a-panel then b-panel
+  constexpr int STAGE = PANEL_A + BN * BIG_ROWB;  // a-panel then b-panel
   constexpr int LA = BM / 64;           // a-panel loads per wave per slab (8 rows x 8 waves each)
-  constexpr int LB = BIG_BN / 64;       // b-panel loads per wave per slab
+  constexpr int LB = BN / 64;           // b-panel loads per wave per slab
   constexpr int H1 = (TM + 1) / 2;      // MFMA rows issued before the next fragments are fetched
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds_big[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -251,7 +249,7 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
     const int rows_in_group = min(tiles_m - first_m, BIG_GROUP_M);
     const int tm_idx = first_m + (pid % group_size) % rows_in_group;
     const int tn_idx = (pid % group_size) / rows_in_group;
-    const int m0 = tm_idx * BM, n0 = tn_idx * BIG_BN;
+    const int m0 = tm_idx * BM, n0 = tn_idx * BN;
 
     uint32_t va[LA], vb[LB];
 #pragma unroll
@@ -287,7 +285,7 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
                                lds_big + (stage ^ 1) * STAGE + PANEL_A + (wave * LB) * 1024,
                                (uint32_t)(kt + 1) * BIG_ROWB);
       const uint8_t* pa = lds_big + stage * STAGE + (wm * WM) * BIG_ROWB;
-      const uint8_t* pb = lds_big + stage * STAGE + PANEL_A + (wn * 64) * BIG_ROWB;
+      const uint8_t* pb = lds_big + stage * STAGE + PANEL_A + (wn * WN) * BIG_ROWB;
       bf16x8_t fa[2][TM], fb[2][TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -332,7 +330,7 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
       __syncthreads();
     }
 
-    // acc[i][j][4 q + e] = out[m0 + wm*WM + i*32 + l32][n0 + wn*64 + j*32 + 8 q + 4 lhi + e]
+    // acc[i][j][4 q + e] = out[m0 + wm*WM + i*32 + l32][n0 + wn*WN + j*32 + 8 q + 4 lhi + e]
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int m = m0 + wm * WM + i * 32 + l32;
@@ -341,7 +339,7 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
       for (int j = 0; j < TN; ++j) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int n = n0 + wn * 64 + j * 32 + 8 * q + 4 * lhi;
+          const int n = n0 + wn * WN + j * 32 + 8 * q + 4 * lhi;
           if (n < N) {
             uint2 v;
             v.x = pack2(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1]);
@@ -355,39 +353,44 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
 }
 
 
-template <int TM>
+template <int TM, int TN>
 static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64_t M, int64_t N,
                       int64_t K, int64_t ldc, int max_cus, hipStream_t hs) {
-  constexpr int BM = 64 * TM;
-  constexpr int LDS = big_lds_bytes(TM);
+  constexpr int BM = 64 * TM, BN = 128 * TN;
+  constexpr int LDS = big_lds_bytes(TM, TN);
   static std::atomic<bool> lds_ok{false};
   if (!lds_ok.load(std::memory_order_acquire)) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_big_kernel<TM>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_big_kernel<TM, TN>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess)
       return set_error(TW_ERR_LAUNCH, "gemm_bf16_nt: the device refused %d bytes of LDS", LDS);
     lds_ok.store(true, std::memory_order_release);
   }
-  const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BIG_BN - 1) / BIG_BN);
+  const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
   int64_t grid = (int64_t)tiles_m * tiles_n;
   if (max_cus > 0 && grid > max_cus) grid = max_cus;
-  hipLaunchKernelGGL(gemm_bf16_nt_big_kernel<TM>, dim3((unsigned)grid), dim3(BIG_THREADS), LDS, hs, out, a,
-                     b, (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n);
+  hipLaunchKernelGGL((gemm_bf16_nt_big_kernel<TM, TN>), dim3((unsigned)grid), dim3(BIG_THREADS), LDS, hs,
+                     out, a, b, (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n);
   return TW_OK;
 }
 
-// Tile height (in 64-row units) that finishes soonest on `cus` compute units: time is
-// proportional to rounds x tile height; ties go to the smaller tile.
-static int pick_tile_height(int64_t M, int64_t N, int cus) {
-  const int64_t tiles_n = (N + BIG_BN - 1) / BIG_BN;
-  int best = 4;
-  int64_t best_cost = INT64_MAX;
-  for (int tm : {3, 4, 5}) {
-    const int64_t tiles = ((M + 64 * tm - 1) / (64 * tm)) * tiles_n;
+// Workgroup tile for the problem, (64 TM) x (128 TN).  Cost = rounds x (tile area + a
+// fixed part per round); ties go to the smaller tile.  Only 64-wide wave tiles (TN = 2)
+// are offered: 96 x 96 wave tiles (192 x 384 workgroup tiles), which read a third
+// fewer LDS fragments per MFMA, measured no faster per tile and fit the compute-unit
+// count worse on the shapes of interest.
+struct BigTile { int tm, tn; };
+
+static BigTile pick_big_tile(int64_t M, int64_t N, int cus) {
+  static const struct { int tm, tn; } kTiles[] = {{3, 2}, {4, 2}, {5, 2}};
+  BigTile best = {4, 2};
+  double best_cost = 1e300;
+  for (const auto& t : kTiles) {
+    const int64_t tiles = ((M + 64 * t.tm - 1) / (64 * t.tm)) * ((N + 128 * t.tn - 1) / (128 * t.tn));
     const int64_t rounds = (tiles + cus - 1) / cus;
-    const int64_t cost = rounds * tm * 64 + 8;  // +8: per-round fixed part (prologue, epilogue)
-    if (cost < best_cost || (cost == best_cost && tm < best)) {
-      best = tm;
+    const double cost = (double)rounds * (64.0 * t.tm * 128.0 * t.tn + 2048.0);
+    if (cost < best_cost) {
       best_cost = cost;
+      best = BigTile{t.tm, t.tn};
     }
   }
   return best;
@@ -417,11 +420,10 @@ int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t
     const uint16_t* pa = static_cast<const uint16_t*>(a);
     const uint16_t* pb = static_cast<const uint16_t*>(b);
     int rc;
-    switch (pick_tile_height(M, N, cus)) {
-      case 3: rc = launch_big<3>(o, pa, pb, M, N, K, ldc, max_cus, hs); break;
-      case 5: rc = launch_big<5>(o, pa, pb, M, N, K, ldc, max_cus, hs); break;
-      default: rc = launch_big<4>(o, pa, pb, M, N, K, ldc, max_cus, hs); break;
-    }
+    const BigTile bt = pick_big_tile(M, N, cus);
+    if (bt.tm == 3) rc = launch_big<3, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
+    else if (bt.tm == 5) rc = launch_big<5, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
+    else rc = launch_big<4, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
     if (rc != TW_OK) return rc;
   } else {
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);

@@ -118,6 +118,35 @@ __device__ __forceinline__ float block_sum(float v, float* slots, int nwaves) {
   return total;
 }
 
+// Maximum of non-negative values: the same DPP steps as wave_sum, then the
+// workgroup's wave maxima through LDS (one slot per wave, at most 16).
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v) {
+  int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true);
+  return fmaxf(v, __int_as_float(moved));
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+  v = dpp_max<0xB1>(v);
+  v = dpp_max<0x4E>(v);
+  v = dpp_max<0x141>(v);
+  v = dpp_max<0x140>(v);
+  float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
+__device__ __forceinline__ float block_max(float v, float* slots, int nwaves) {
+  v = wave_max(v);
+  if (nwaves == 1) return v;
+  const int lane = threadIdx.x & 63;
+  if (lane == 0) slots[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return wave_max(lane < nwaves ? slots[lane] : 0.0f);
+}
+
 constexpr int kMaxChunks = 64;  // 4096 vectors = hidden size 32768
 
 template <int VPT>
@@ -181,6 +210,44 @@ __device__ __forceinline__ uint32_t quant4_fp8(float a, float b, float c, float 
   return (uint32_t)r;
 }
 
+// Output kinds.  Static fp8 quantises the bf16 result of the unquantised op with a
+// caller-supplied scale.  The two dynamic kinds follow the reference's fused kernel
+// (csrc/quantization/fused_kernels/layernorm_utils.cuh:51-124): the normalised value
+// is n = bf16(bf16(s * inv) * w) computed from the unrounded fp32 sum s, the row's
+// scale is max(min(max|n|, ub) / qmax, floor), and the codes are
+// fp8(clamp(n / scale)) or int8(sat(rint(n * (1 / scale)))).
+constexpr int kQNone = 0, kQStaticFp8 = 1, kQDynFp8 = 2, kQDynInt8 = 3;
+constexpr float kFp8MinScale = 1.0f / (448.0f * 512.0f);  // csrc/quantization/utils.cuh:48-52
+constexpr float kInt8MinScale = 1.1920928955078125e-07f;  // FLT_EPSILON, utils.cuh:55-59
+
+__device__ __forceinline__ float dyn_scale(float amax, const float* scale_ub, bool int8) {
+  float sc = scale_ub ? fminf(amax, *scale_ub) : amax;
+  return int8 ? fmaxf(sc / 127.0f, kInt8MinScale) : fmaxf(sc / kFp8Max, kFp8MinScale);
+}
+
+// Four values -> four fp8 codes, true division by the scale
+// (quant_conversions.cuh:34-39,62-69).
+__device__ __forceinline__ uint32_t quant4_fp8_div(float a, float b, float c, float d, float scale) {
+  a = fmaxf(-kFp8Max, fminf(a / scale, kFp8Max));
+  b = fmaxf(-kFp8Max, fminf(b / scale, kFp8Max));
+  c = fmaxf(-kFp8Max, fminf(c / scale, kFp8Max));
+  d = fmaxf(-kFp8Max, fminf(d / scale, kFp8Max));
+  int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+  return (uint32_t)r;
+}
+
+// Round to nearest even, saturate (quant_conversions.cuh:14-32).
+__device__ __forceinline__ uint32_t quant1_int8(float x, float scale_inv) {
+  float q = fmaxf(-128.0f, fminf(__builtin_rintf(x * scale_inv), 127.0f));
+  return (uint32_t)(int)q & 0xffu;
+}
+
+__device__ __forceinline__ uint32_t quant4_int8(float a, float b, float c, float d, float scale_inv) {
+  return quant1_int8(a, scale_inv) | (quant1_int8(b, scale_inv) << 8) |
+         (quant1_int8(c, scale_inv) << 16) | (quant1_int8(d, scale_inv) << 24);
+}
+
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ void store8(__amdgpu_buffer_rsrc_t d, uint32_t off, uint32_t lo, uint32_t hi) {
   u32x2_t t = {lo, hi};
@@ -203,12 +270,16 @@ __device__ __forceinline__ void store16(__amdgpu_buffer_rsrc_t d, uint32_t off, 
 // y may alias any partial: a lane stores y only to vector slots it has already
 // read in every buffer.  blockDim.x must be a multiple of 64.
 // ---------------------------------------------------------------------------
-template <int NP, int VPT, int MAXNT, bool HAS_RES, bool COPY, bool FP8>
+//   Q        output kind (kQNone .. kQDynInt8); quant_scale is the static scale
+//            (kQStaticFp8) or the optional upper bound of the row scale (kQDynFp8)
+template <int NP, int VPT, int MAXNT, bool HAS_RES, bool COPY, int Q>
 __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
     PartialPtrs parts, int np_rt, void* y_out, void* residual, void* copy_out,
-    const void* __restrict__ weight, const float* __restrict__ quant_scale, float eps,
-    int num_tokens, int vec_per_row, float hidden) {
+    const void* __restrict__ weight, const float* __restrict__ quant_scale,
+    float* __restrict__ row_scales, float eps, int num_tokens, int vec_per_row, float hidden) {
+  constexpr bool FP8 = Q == kQStaticFp8;
   __shared__ float slots[2][kMaxChunks];
+  __shared__ float max_slots[2][16];
   const int nt = blockDim.x;
   const int nwaves = nt >> 6;
   const int nchunks = (vec_per_row + 63) >> 6;  // <= VPT * nwaves
@@ -303,7 +374,45 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
 
     // bf16 output: 16 bytes per vector; fp8 output: the bf16 result quantised, 8 bytes
     // per vector in rows of half the size.
-    const __amdgpu_buffer_rsrc_t dy = row_desc(y_out, row, FP8 ? row_bytes / 2 : row_bytes);
+    const __amdgpu_buffer_rsrc_t dy = row_desc(y_out, row, Q != kQNone ? row_bytes / 2 : row_bytes);
+    if (Q == kQDynFp8 || Q == kQDynInt8) {
+      uint4 nv[VPT];
+      float amax = 0.0f;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        float w[8], t[8];
+        unpack8(wv[k], w);
+        uint4 tv;
+        tv.x = pack_bf16(s[k][0] * inv, s[k][1] * inv);
+        tv.y = pack_bf16(s[k][2] * inv, s[k][3] * inv);
+        tv.z = pack_bf16(s[k][4] * inv, s[k][5] * inv);
+        tv.w = pack_bf16(s[k][6] * inv, s[k][7] * inv);
+        unpack8(tv, t);
+        nv[k].x = pack_bf16(t[0] * w[0], t[1] * w[1]);
+        nv[k].y = pack_bf16(t[2] * w[2], t[3] * w[3]);
+        nv[k].z = pack_bf16(t[4] * w[4], t[5] * w[5]);
+        nv[k].w = pack_bf16(t[6] * w[6], t[7] * w[7]);
+        unpack8(nv[k], t);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(t[e]));
+      }
+      amax = block_max(amax, max_slots[phase], nwaves);
+      const float scale = dyn_scale(amax, quant_scale, Q == kQDynInt8);
+      if (threadIdx.x == 0) row_scales[row] = scale;
+      const float sinv = 1.0f / scale;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        float n[8];
+        unpack8(nv[k], n);
+        if (Q == kQDynInt8)
+          store8(dy, off[k] / 2, quant4_int8(n[0], n[1], n[2], n[3], sinv),
+                 quant4_int8(n[4], n[5], n[6], n[7], sinv));
+        else
+          store8(dy, off[k] / 2, quant4_fp8_div(n[0], n[1], n[2], n[3], scale),
+                 quant4_fp8_div(n[4], n[5], n[6], n[7], scale));
+      }
+      continue;
+    }
     float scale_inv = 1.0f;
     if (FP8) scale_inv = 1.0f / *quant_scale;
 #pragma unroll
@@ -394,6 +503,61 @@ __global__ __launch_bounds__(1024) void row_norm_elem_kernel(
   }
 }
 
+// Element-wise kernel with dynamic per-token quantisation: three passes over the
+// row, like the reference's scalar path (layernorm_utils.cuh:19-124) — sum of
+// squares, row maximum of the normalised value, quantise (+ residual write-back).
+// The sum is recomputed from the inputs in every pass: the residual is overwritten
+// only in the last one, by the lane that read it.
+template <typename T, bool HAS_RES, bool INT8>
+__global__ __launch_bounds__(1024) void row_norm_dyn_elem_kernel(
+    PartialPtrs parts, int np, uint8_t* out, float* __restrict__ row_scales, T* residual,
+    const T* __restrict__ weight, const float* __restrict__ scale_ub, float eps, int num_tokens,
+    int hidden_size) {
+  __shared__ float slots[2][16];
+  __shared__ float max_slots[2][16];
+  const int tid = threadIdx.x;
+  const int nt = blockDim.x;
+  const int nwaves = nt >> 6;
+  int phase = 0;
+  for (int row = blockIdx.x; row < num_tokens; row += gridDim.x, phase ^= 1) {
+    const size_t base = (size_t)row * hidden_size;
+    auto sum_at = [&](int j) {
+      float s = Elem<T>::load(static_cast<const T*>(parts.p[0]) + base + j);
+      for (int p = 1; p < np; ++p) s += Elem<T>::load(static_cast<const T*>(parts.p[p]) + base + j);
+      if (HAS_RES) s += Elem<T>::load(residual + base + j);
+      return s;
+    };
+    auto normed = [&](float s, float inv, int j) {
+      const T t = Elem<T>::round(s * inv);
+      const T n = Elem<T>::round(Elem<T>::load(&t) * Elem<T>::load(weight + j));
+      return Elem<T>::load(&n);
+    };
+    float ss = 0.0f;
+    for (int j = tid; j < hidden_size; j += nt) {
+      const float s = sum_at(j);
+      ss += s * s;
+    }
+    const float inv = inv_rms(block_sum(ss, slots[phase], nwaves), (float)hidden_size, eps);
+    float amax = 0.0f;
+    for (int j = tid; j < hidden_size; j += nt) amax = fmaxf(amax, fabsf(normed(sum_at(j), inv, j)));
+    amax = block_max(amax, max_slots[phase], nwaves);
+    const float scale = dyn_scale(amax, scale_ub, INT8);
+    if (tid == 0) row_scales[row] = scale;
+    const float sinv = 1.0f / scale;
+    for (int j = tid; j < hidden_size; j += nt) {
+      const float s = sum_at(j);
+      if (HAS_RES) residual[base + j] = Elem<T>::round(s);
+      const float n = normed(s, inv, j);
+      if (INT8) {
+        out[base + j] = (uint8_t)quant1_int8(n, sinv);
+      } else {
+        const float q = fmaxf(-kFp8Max, fminf(n / scale, kFp8Max));
+        out[base + j] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(q, q, 0, false) & 0xff);
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
@@ -444,23 +608,25 @@ struct RowNormArgs {
   void* residual;
   void* copy_out;
   const void* weight;
-  const float* quant_scale;  // non-null: y is fp8 (e4m3fn), quantised with this device scalar
+  int q;                     // output kind (kQNone ..)
+  const float* quant_scale;  // static fp8: the scale; dynamic fp8: optional upper bound (may be null)
+  float* row_scales;         // dynamic kinds: one scale per row (output)
   int64_t T, H;
   float eps;
   int grid;
   hipStream_t stream;
 };
 
-template <int NP, bool HAS_RES, bool COPY, bool FP8>
+template <int NP, bool HAS_RES, bool COPY, int Q>
 static int launch_vec(const RowNormArgs& a) {
   const int V = (int)(a.H / 8);
   VecShape sh;
   if (!vec_shape(V, a.T, &sh)) return 1;  // caller falls back to the element-wise kernel
   dim3 g(a.grid), b(sh.nt);
 #define TW_LAUNCH(VPT, MAXNT)                                                                    \
-  hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, MAXNT, HAS_RES, COPY, FP8>), g, b, 0,        \
+  hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, MAXNT, HAS_RES, COPY, Q>), g, b, 0,          \
                      a.stream, a.parts, a.np, a.y, a.residual, a.copy_out, a.weight,             \
-                     a.quant_scale, a.eps, (int)a.T, V, (float)a.H)
+                     a.quant_scale, a.row_scales, a.eps, (int)a.T, V, (float)a.H)
   if (sh.vpt == 1) TW_LAUNCH(1, 1024);
   else if (sh.vpt == 2) TW_LAUNCH(2, 1024);
   else if (sh.maxnt == 256) TW_LAUNCH(4, 256);
@@ -471,13 +637,26 @@ static int launch_vec(const RowNormArgs& a) {
 
 // mode: residual given -> add + write back; copy_out given -> rms_norm_inplace;
 // neither -> rms_norm.  Only the P = 1 kernels exist without a residual.
+template <int NP, bool HAS_RES>
+static int launch_vec_q(const RowNormArgs& a) {
+  switch (a.q) {
+    case kQNone: return launch_vec<NP, HAS_RES, false, kQNone>(a);
+    case kQStaticFp8: return launch_vec<NP, HAS_RES, false, kQStaticFp8>(a);
+    case kQDynFp8: return launch_vec<NP, HAS_RES, false, kQDynFp8>(a);
+    default: return launch_vec<NP, HAS_RES, false, kQDynInt8>(a);
+  }
+}
+
 template <int NP>
 static int launch_vec_mode(const RowNormArgs& a) {
-  const bool fp8 = a.quant_scale != nullptr;
-  if (a.residual) return fp8 ? launch_vec<NP, true, false, true>(a) : launch_vec<NP, true, false, false>(a);
-  if (NP != 1) return 1;
-  if (a.copy_out) return fp8 ? 1 : launch_vec<1, false, true, false>(a);
-  return fp8 ? launch_vec<1, false, false, true>(a) : launch_vec<1, false, false, false>(a);
+  if (a.residual) return launch_vec_q<NP, true>(a);
+  if (a.copy_out) return (NP == 1 && a.q == kQNone) ? launch_vec<1, false, true, kQNone>(a) : 1;
+  // Without a residual only P = 1 and the dynamic kinds (whose P-partial form may come
+  // without one) have vector kernels.
+  if (NP == 1) return launch_vec_q<1, false>(a);
+  if (a.q == kQDynFp8) return launch_vec<NP, false, false, kQDynFp8>(a);
+  if (a.q == kQDynInt8) return launch_vec<NP, false, false, kQDynInt8>(a);
+  return 1;
 }
 
 template <typename T>
@@ -488,7 +667,17 @@ static void launch_elem(const RowNormArgs& a) {
   hipLaunchKernelGGL((row_norm_elem_kernel<T, HAS_RES, COPY, FP8>), g, b, 0, a.stream, a.parts,  \
                      a.np, a.y, static_cast<T*>(a.residual), static_cast<T*>(a.copy_out),        \
                      static_cast<const T*>(a.weight), a.quant_scale, a.eps, (int)a.T, (int)a.H)
-  const bool fp8 = a.quant_scale != nullptr;
+  if (a.q == kQDynFp8 || a.q == kQDynInt8) {
+#define TW_LAUNCH_DYN(HAS_RES, INT8)                                                             \
+  hipLaunchKernelGGL((row_norm_dyn_elem_kernel<T, HAS_RES, INT8>), g, b, 0, a.stream, a.parts,   \
+                     a.np, static_cast<uint8_t*>(a.y), a.row_scales, static_cast<T*>(a.residual), \
+                     static_cast<const T*>(a.weight), a.quant_scale, a.eps, (int)a.T, (int)a.H)
+    if (a.residual) { if (a.q == kQDynInt8) TW_LAUNCH_DYN(true, true); else TW_LAUNCH_DYN(true, false); }
+    else { if (a.q == kQDynInt8) TW_LAUNCH_DYN(false, true); else TW_LAUNCH_DYN(false, false); }
+#undef TW_LAUNCH_DYN
+    return;
+  }
+  const bool fp8 = a.q == kQStaticFp8;
   if (a.residual) { if (fp8) TW_LAUNCH(true, false, true); else TW_LAUNCH(true, false, false); }
   else if (a.copy_out) TW_LAUNCH(false, true, false);
   else { if (fp8) TW_LAUNCH(false, false, true); else TW_LAUNCH(false, false, false); }
@@ -503,13 +692,15 @@ static int finish_launch(const char* what) {
 }
 
 // Shared by every entry point.  residual == nullptr: no residual add;
-// copy_out != nullptr: rms_norm_inplace; quant_scale != nullptr: y is fp8.
+// copy_out != nullptr: rms_norm_inplace; quant: 0 = y in the input's type, 1 = fp8
+// with the static scale *quant_scale, 2 / 3 = dynamic per-token fp8 / int8 (row scales
+// to row_scales, quant_scale = optional upper bound).
 // require_vec: refuse instead of falling back to the element-wise kernel (the
 // *_cta contract).
-int run_row_norm(const char* what, const void* const* partials, int np, void* y,
-                 void* residual, void* copy_out, const void* weight, const float* quant_scale,
-                 int64_t T, int64_t H, float eps, int dtype, int max_ctas, bool require_vec,
-                 void* stream_v) {
+int run_row_norm_q(const char* what, const void* const* partials, int np, void* y,
+                   void* residual, void* copy_out, const void* weight, int quant,
+                   const float* quant_scale, float* row_scales, int64_t T, int64_t H, float eps,
+                   int dtype, int max_ctas, bool require_vec, void* stream_v) {
   if (np < 1 || np > TW_MAX_PARTIALS)
     return set_error(TW_ERR_INVALID_ARGUMENT, "%s: number of partials %d not in [1, %d]", what, np,
                      TW_MAX_PARTIALS);
@@ -521,8 +712,15 @@ int run_row_norm(const char* what, const void* const* partials, int np, void* y,
   if (T == 0) return TW_OK;
   if (!y || !weight || !partials)
     return set_error(TW_ERR_INVALID_ARGUMENT, "%s: null pointer argument", what);
-  if (quant_scale && copy_out)
-    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: fp8 output is not defined for the in-place op", what);
+  if (quant < kQNone || quant > kQDynInt8)
+    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: unknown output kind %d", what, quant);
+  if (quant != kQNone && copy_out)
+    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: quantised output is not defined for the in-place op", what);
+  if ((quant == kQStaticFp8 && !quant_scale) || (quant >= kQDynFp8 && !row_scales))
+    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: scale pointer is null", what);
+  if (quant == kQDynInt8 && quant_scale)
+    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: an upper bound of the scale is defined for fp8 output only",
+                     what);
   RowNormArgs a = {};
   bool aligned = aligned16(y) && aligned16(weight) && (!residual || aligned16(residual)) &&
                  (!copy_out || aligned16(copy_out));
@@ -533,7 +731,7 @@ int run_row_norm(const char* what, const void* const* partials, int np, void* y,
     aligned = aligned && aligned16(partials[p]);
   }
   // fp8 rows are H bytes: H % 16 keeps every row of the output 16-byte aligned too
-  const bool vec_ok = aligned && (H % 8 == 0) && (!quant_scale || H % 16 == 0);
+  const bool vec_ok = aligned && (H % 8 == 0) && (quant == kQNone || H % 16 == 0);
   if (require_vec && (!vec_ok || dtype != TW_DTYPE_BF16)) {
     if (dtype != TW_DTYPE_BF16)
       return set_error(TW_ERR_DTYPE, "%s: only bf16 is supported", what);
@@ -549,7 +747,9 @@ int run_row_norm(const char* what, const void* const* partials, int np, void* y,
   a.residual = residual;
   a.copy_out = copy_out;
   a.weight = weight;
+  a.q = quant;
   a.quant_scale = quant_scale;
+  a.row_scales = row_scales;
   a.T = T;
   a.H = H;
   a.eps = eps;
@@ -575,6 +775,15 @@ int run_row_norm(const char* what, const void* const* partials, int np, void* y,
     default: launch_elem<float>(a); break;
   }
   return finish_launch(what);
+}
+
+int run_row_norm(const char* what, const void* const* partials, int np, void* y,
+                 void* residual, void* copy_out, const void* weight, const float* quant_scale,
+                 int64_t T, int64_t H, float eps, int dtype, int max_ctas, bool require_vec,
+                 void* stream) {
+  return run_row_norm_q(what, partials, np, y, residual, copy_out, weight,
+                        quant_scale ? kQStaticFp8 : kQNone, quant_scale, nullptr, T, H, eps, dtype,
+                        max_ctas, require_vec, stream);
 }
 
 // ---------------------------------------------------------------------------

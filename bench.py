@@ -70,7 +70,7 @@ class NormRunner:
     """Pre-binds the C-ABI call for each input set so the timed loop is one ctypes
     call per step (argument checks were done once, here, by the regular shim)."""
 
-    def __init__(self, cfg, nsets, max_ctas, device):
+    def __init__(self, cfg, nsets, max_ctas, device, epilogue="bf16"):
         import torch
         from tokenweave_amd import _custom_ops as ops
         from tokenweave_amd import _lib
@@ -87,8 +87,34 @@ class NormRunner:
             self.sets.append((inp, ptrs))
             self.calls.append((ptrs, cfg.P, out.data_ptr(), inp.residual.data_ptr(),
                                inp.weight.data_ptr(), cfg.T, cfg.H, max_ctas, cfg.eps))
+            if epilogue != "bf16":
+                self._bind_quant(i, epilogue, inp, ptrs, max_ctas, device)
         torch.cuda.synchronize()
-        self.fn = self.lib.tw_reduce_add_rms_norm
+        self.fn = {"bf16": self.lib.tw_reduce_add_rms_norm,
+                   "fp8_static": self.lib.tw_reduce_add_rms_norm_static_fp8_quant,
+                   "fp8_dynamic": self.lib.tw_reduce_add_rms_norm_dynamic_per_token_quant,
+                   "int8_dynamic": self.lib.tw_reduce_add_rms_norm_dynamic_per_token_quant}[epilogue]
+
+    def _bind_quant(self, i, epilogue, inp, ptrs, max_ctas, device):
+        """Replaces call i by the same reduction with a quantised output (one byte per
+        element into its own buffer, a float per row for the dynamic kinds)."""
+        torch, cfg = self.torch, self.cfg
+        from tokenweave_amd import _custom_ops as ops
+        qdtype = torch.int8 if epilogue == "int8_dynamic" else torch.float8_e4m3fn
+        out = torch.empty(cfg.T, cfg.H, dtype=qdtype, device=device)
+        scales = torch.full((max(cfg.T, 1), 1), 0.05, dtype=torch.float32, device=device)
+        self.sets[i] = self.sets[i] + (out, scales)
+        if epilogue == "fp8_static":
+            ops.reduce_add_rms_norm_static_fp8_quant(inp.partials, out, inp.residual, inp.weight,
+                                                     scales[:1].reshape(1), cfg.eps, max_ctas or None)
+            self.calls[i] = (ptrs, cfg.P, out.data_ptr(), inp.residual.data_ptr(), inp.weight.data_ptr(),
+                             scales.data_ptr(), cfg.T, cfg.H, max_ctas, cfg.eps)
+        else:
+            ops.reduce_add_rms_norm_dynamic_per_token_quant(inp.partials, out, scales, inp.residual,
+                                                            inp.weight, cfg.eps, None, max_ctas or None)
+            self.calls[i] = (ptrs, cfg.P, out.data_ptr(), scales.data_ptr(), inp.residual.data_ptr(),
+                             inp.weight.data_ptr(), None, cfg.T, cfg.H, max_ctas, cfg.eps,
+                             1 if epilogue == "int8_dynamic" else 0)
 
     def step(self, i, stream_ptr):
         rc = self.fn(*self.calls[i % len(self.calls)], stream_ptr)
@@ -96,7 +122,13 @@ class NormRunner:
             raise RuntimeError(self.lib.tw_last_error().decode())
 
 
-def time_norm(cfg, steps, warmup, max_ctas, device):
+def quant_bytes(cfg, epilogue):
+    """Algorithmic bytes with a quantised output: one byte per element instead of two,
+    plus one float per row for the dynamic kinds."""
+    return cfg.bytes - cfg.T * cfg.H + (4 * cfg.T if epilogue.endswith("dynamic") else 4)
+
+
+def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16"):
     """Returns dict(ms_per_step, gbps, kernel_us_mean): wall-clock per step between the
     two synchronisation points, and the mean launch duration from the HIP events that
     bracket the same `steps` back-to-back launches."""
@@ -105,7 +137,7 @@ def time_norm(cfg, steps, warmup, max_ctas, device):
     free, _ = torch.cuda.mem_get_info()
     set_bytes = (cfg.P + 1) * cfg.T * cfg.H * 2 + cfg.H * 2
     nsets = max(2, min(nsets, int(free * 0.6) // (set_bytes * 3)))  # fp32 staging while generating
-    runner = NormRunner(cfg, nsets, max_ctas, device)
+    runner = NormRunner(cfg, nsets, max_ctas, device, epilogue)
     stream = torch.cuda.current_stream()
     sp = ctypes.c_void_p(stream.cuda_stream)
     for i in range(warmup):
@@ -304,7 +336,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name) if args.max_ctas == 0 else None,
-                     "kernel": "row_norm_bf16_kernel<8,4,256,true,false>",
+                     "kernel": "row_norm_bf16_kernel<8,4,256,true,false,0>",
                      "kernel_us_mean": round(kernel_us, 3)},
     }
     if not args.no_cpu_baseline:
@@ -327,6 +359,16 @@ def main():
                            "gbps": round(c.bytes / r["kernel_us_mean"] / 1e3, 1),
                            "pct_hbm_peak": round(c.bytes / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
             log(f"[sweep] {name}: {sweep[name]}")
+        for name in ("c2_llama70b_tp8_shard@T256", "c2_unsharded@T2048"):
+            c = cfgs[name]
+            steps = max(50, min(2000, int(0.02 * 5e12 / c.bytes)))
+            for epi in ("fp8_static", "fp8_dynamic", "int8_dynamic"):
+                r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device, epi)
+                b = quant_bytes(c, epi)
+                sweep[f"{name}+{epi}"] = {"bytes": b, "kernel_us": round(r["kernel_us_mean"], 3),
+                                          "gbps": round(b / r["kernel_us_mean"] / 1e3, 1),
+                                          "pct_hbm_peak": round(b / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
+                log(f"[sweep] {name}+{epi}: {sweep[f'{name}+{epi}']}")
         w = time_weave(device, norm_cap=0, gemm_cap=128)
         sweep["c5_weave"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}
         log(f"[sweep] c5_weave: {sweep['c5_weave']}")

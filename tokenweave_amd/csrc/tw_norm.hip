@@ -290,6 +290,10 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
   for (int k = 0; k < VPT; ++k) off[k] = (threadIdx.x + k * nt) * 16u;
 
   const __amdgpu_buffer_rsrc_t dw = row_desc(weight, 0, row_bytes);
+  // The static scale / the optional bound of the dynamic scale: one scalar, read ahead
+  // of the row loop so that its latency is not behind the reduction.
+  float qparam = __builtin_inff();
+  if (Q != kQNone && quant_scale) qparam = *quant_scale;
 
   int phase = 0;
   for (int row = blockIdx.x; row < num_tokens; row += gridDim.x, phase ^= 1) {
@@ -397,7 +401,7 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
         for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(t[e]));
       }
       amax = block_max(amax, max_slots[phase], nwaves);
-      const float scale = dyn_scale(amax, quant_scale, Q == kQDynInt8);
+      const float scale = dyn_scale(fminf(amax, qparam), nullptr, Q == kQDynInt8);
       if (threadIdx.x == 0) row_scales[row] = scale;
       const float sinv = 1.0f / scale;
 #pragma unroll
@@ -413,8 +417,7 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
       }
       continue;
     }
-    float scale_inv = 1.0f;
-    if (FP8) scale_inv = 1.0f / *quant_scale;
+    const float scale_inv = 1.0f / qparam;
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       float r[8], w[8];

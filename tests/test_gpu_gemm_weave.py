@@ -71,6 +71,26 @@ def test_gemm_output_with_wide_row_stride():
     assert not wide[:, 128:].any()
 
 
+@pytest.mark.parametrize("M,N,K,ldc,shift", [
+    (300, 256, 128, 512, 0),    # 16-byte stores into a slice of a wider buffer
+    (300, 388, 128, 388, 0),    # N % 8 != 0: 8-byte stores
+    (300, 384, 128, 388, 0),    # row stride % 8 != 0: 8-byte stores
+    (300, 384, 128, 384, 4),    # out 8-byte but not 16-byte aligned: 8-byte stores
+    (645, 520, 192, 520, 0),    # ragged tile edges in both directions, 16-byte stores
+])
+def test_gemm_large_tile_kernel_store_paths(M, N, K, ldc, shift):
+    print(f"[case] gemm stores M={M} N={N} K={K} ldc={ldc} shift={shift}", flush=True)
+    g = wl.make_gemm_inputs(M, N, K, DEV, seed=M + N + ldc + shift)
+    flat = torch.zeros(M * ldc + 16, dtype=torch.bfloat16, device=DEV)
+    out = flat[shift:shift + M * ldc].view(M, ldc)[:, :N]
+    ops.gemm_bf16_nt(out, g.a, g.b)
+    torch.cuda.synchronize()
+    check(out, g.a, g.b, "store path")
+    if ldc > N:
+        assert not flat[shift:shift + M * ldc].view(M, ldc)[:, N:].any(), "columns past N were written"
+    assert not flat[:shift].any() and not flat[shift + M * ldc:].any()
+
+
 def test_weave_step_equals_serial_execution():
     """GEMM of split A on the current stream while split B's fused norm runs on a
     second stream (tokenweave_utils.py:236-260): same bits as running them in turn."""

@@ -7,7 +7,9 @@
 // Both operands are K-contiguous, so the 8 consecutive k a lane feeds to
 // v_mfma_f32_32x32x16_bf16 are one 16-byte chunk of a row of `a` or `b`.  The
 // MFMA is issued with `b` rows as its first operand, which leaves every lane
-// with 4 consecutive n per accumulator quad: 8-byte row-major stores.
+// with 4 consecutive n per accumulator quad: 8-byte row-major stores, or, in the
+// big kernel when the output allows 16-byte stores, a transpose through LDS into
+// whole 128-byte lines per row.
 //
 // Two kernels:
 //  * gemm_bf16_nt_big_kernel<TM> (K % 64 == 0): (64 TM) x 256 x 64 tiles, TM = 3,
@@ -205,7 +207,7 @@ __device__ __forceinline__ void big_issue_slab(__amdgpu_buffer_rsrc_t da, __amdg
 template <int TM, int TN>
 __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
-    int M, int N, int K, int64_t ldc, int tiles_m, int tiles_n) {
+    int M, int N, int K, int64_t ldc, int tiles_m, int tiles_n, int wide_store) {
   constexpr int WM = 32 * TM, WN = 32 * TN;  // wave tile
   constexpr int BM = 2 * WM, BN = 4 * WN;    // workgroup tile: the 8 waves as 2 x 4
   constexpr int PANEL_A = BM * BIG_ROWB;
@@ -331,6 +333,49 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
     }
 
     // acc[i][j][4 q + e] = out[m0 + wm*WM + i*32 + l32][n0 + wn*WN + j*32 + 8 q + 4 lhi + e]
+    if (wide_store) {
+      // Through LDS, 32 rows of the wave tile at a time (a wave-private 32 x WN patch,
+      // rows padded by 8 bytes): lanes write their 4-element groups, then read the patch
+      // back row-contiguously, 16 bytes per lane, so that a wave store covers whole
+      // 128-byte lines of 8 output rows instead of 16-byte pieces of 32 rows.  The slab
+      // stages are free: every wave passed the barrier that ends the k loop.
+      constexpr int PATCH_ROW = WN * 2 + 8;            // bytes
+      constexpr int CHUNKS = WN / 8;                   // 16-byte chunks per patch row
+      constexpr int ROWS_PER_PASS = 64 / CHUNKS;
+      static_assert(64 % CHUNKS == 0 && 32 % ROWS_PER_PASS == 0, "patch read-back shape");
+      uint8_t* patch = lds_big + wave * (32 * PATCH_ROW);
+      const int rd_row = lane / CHUNKS, rd_chunk = lane % CHUNKS;
+      const int n = n0 + wn * WN + rd_chunk * 8;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            uint2 v;
+            v.x = pack2(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1]);
+            v.y = pack2(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+            *reinterpret_cast<uint2*>(patch + l32 * PATCH_ROW + (j * 32 + 8 * q + 4 * lhi) * 2) = v;
+          }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int r = 0; r < 32; r += ROWS_PER_PASS) {
+          const int row = r + rd_row;
+          const int m = m0 + wm * WM + i * 32 + row;
+          // 8-byte LDS reads: the padded row pitch keeps rows 8-byte, not 16-byte, aligned
+          const uint2 lo = *reinterpret_cast<const uint2*>(patch + row * PATCH_ROW + rd_chunk * 16);
+          const uint2 hi = *reinterpret_cast<const uint2*>(patch + row * PATCH_ROW + rd_chunk * 16 + 8);
+          if (m < M && n < N)
+            *reinterpret_cast<uint4*>(out + (size_t)m * ldc + n) = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+      continue;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int m = m0 + wm * WM + i * 32 + l32;
@@ -352,7 +397,6 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
   }
 }
 
-
 template <int TM, int TN>
 static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64_t M, int64_t N,
                       int64_t K, int64_t ldc, int max_cus, hipStream_t hs) {
@@ -368,8 +412,10 @@ static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
   int64_t grid = (int64_t)tiles_m * tiles_n;
   if (max_cus > 0 && grid > max_cus) grid = max_cus;
+  // 16-byte stores need 16-byte aligned row segments that end inside the row
+  const int wide_store = (N % 8 == 0 && ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) ? 1 : 0;
   hipLaunchKernelGGL((gemm_bf16_nt_big_kernel<TM, TN>), dim3((unsigned)grid), dim3(BIG_THREADS), LDS, hs,
-                     out, a, b, (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n);
+                     out, a, b, (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n, wide_store);
   return TW_OK;
 }
 

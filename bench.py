@@ -43,7 +43,7 @@ ROTATION_BYTES = 4 << 30      # distinct operand bytes cycled through before any
 # WRITE_SIZE, each scaled by the same counter's reading for the library's plain copy
 # kernel of known size); the runs are summarised in
 # profiles/row_norm_bf16_c2_T256_pmc_traffic.md.  Workloads without a counter run: None.
-MEASURED_TRAFFIC_BYTES = {"c2_llama70b_tp8_shard@T256": 46373129}
+MEASURED_TRAFFIC_BYTES = {"c2_llama70b_tp8_shard@T256": 46366607}
 
 
 def log(*a):

@@ -187,7 +187,7 @@ TW_API int tw_reduce_add_rms_norm_static_fp8_quant(const void* const* partials, 
  * out: [num_tokens, hidden_size] bytes; scales: num_tokens floats (device);
  * scale_ub: NULL or one device float (fp8 only); residual: NULL or
  * [num_tokens, hidden_size], updated in place.  input is not modified.  Any
- * hidden_size / alignment (vector kernel for bf16, 16-byte aligned, hidden_size % 16 == 0).
+ * hidden_size / alignment (vector kernel for bf16 and fp16, 16-byte aligned, hidden_size % 16 == 0).
  * Replaces ::rms_norm_dynamic_per_token_quant
  * (csrc/quantization/fused_kernels/fused_layernorm_dynamic_per_token_quant.cu:131-155,
  * schema at csrc/torch_bindings.cpp:216-221). */

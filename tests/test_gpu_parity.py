@@ -108,6 +108,54 @@ def test_reference_unit_test_grid(num_tokens, hidden_size, add_residual, dtype):
         torch.testing.assert_close(out, ref_out, atol=1e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("T,H", [(7, 8), (83, 768), (300, 5120), (40, 8192), (1000, 8192), (5, 16384), (3, 32768)])
+@pytest.mark.parametrize("op", ["fused_add", "rms_norm", "inplace"])
+def test_fp16_vector_kernel_tight(T, H, op):
+    """fp16 tensors take the 16-byte vector kernel when aligned.  Same arithmetic as
+    bf16: residual = one RNE rounding of the fp32 sum (exact to check), output = one
+    rounding of f32(residual) * inv * f32(w) — compared with float64 arithmetic to one
+    fp16 step, and with the element-wise kernel (reached through a 2-byte-shifted,
+    hence unaligned, copy of the same data) to one step on few elements."""
+    torch.manual_seed(T + H)
+    x = torch.randn(T, H, device=DEV).half()
+    r = torch.randn(T, H, device=DEV).half()
+    w = (1 + 0.1 * torch.randn(H, device=DEV)).half()
+    eps = 1e-5
+
+    def shifted(t):   # same values at an address that is 2 bytes off 16-byte alignment
+        flat = torch.empty(t.numel() + 8, dtype=t.dtype, device=DEV)
+        v = flat[1:1 + t.numel()].view(t.shape)
+        v.copy_(t)
+        return v
+
+    def run(xx, rr, ww):
+        if op == "fused_add":
+            ops.fused_add_rms_norm(xx, rr, ww, eps)
+            return xx, rr
+        out = torch.empty_like(xx) if xx.data_ptr() % 16 == 0 else shifted(xx)
+        if op == "rms_norm":
+            ops.rms_norm(out, xx, ww, eps)
+            return out, None
+        ops.rms_norm_inplace(out, xx, ww, eps)   # out <- x ; x <- norm(x)
+        return xx, out
+
+    s32 = x.float() + r.float() if op == "fused_add" else x.float()
+    src = s32.half()
+    inv = 1.0 / torch.sqrt((s32.double() ** 2).mean(dim=-1, keepdim=True) + eps)
+    y64 = src.double() * inv * w.double()
+    y_vec, aux_vec = run(x.clone(), r.clone(), w)
+    y_el, aux_el = run(shifted(x), shifted(r), shifted(w))
+    torch.cuda.synchronize()
+    if op == "fused_add":
+        assert torch.equal(aux_vec, src) and torch.equal(aux_el, src)
+    if op == "inplace":
+        assert torch.equal(aux_vec, x) and torch.equal(aux_el, x)
+    step = torch.maximum(y64.abs() * 2.0 ** -10, torch.tensor(2.0 ** -24, device=DEV, dtype=torch.float64))
+    assert bool(((y_vec.double() - y64).abs() <= step).all())
+    d = (y_vec.view(torch.int16).int() - y_el.view(torch.int16).int()).abs()
+    assert int(d.max()) <= 1 and float((d != 0).float().mean()) <= 2e-3
+
+
 @pytest.mark.parametrize("T,H", [(7, 8), (83, 768), (83, 5120), (4096, 8192), (5, 16384), (3, 32768), (2, 40960)])
 def test_bf16_grid_against_checker_tight(oracle, T, H):
     torch.manual_seed(1)

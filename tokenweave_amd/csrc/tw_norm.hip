@@ -71,6 +71,41 @@ __device__ __forceinline__ void add8(const uint4& v, float (&f)[8]) {
   f[6] += bf16_lo(v.w); f[7] += bf16_hi(v.w);
 }
 
+// The vector kernel's view of a 16-bit element type: widen a 32-bit word (element
+// 2i in the low half) and narrow two floats with round-to-nearest-even.
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+template <typename E> struct Pk;
+template <> struct Pk<__bf16> {
+  static __device__ __forceinline__ float lo(uint32_t u) { return bf16_lo(u); }
+  static __device__ __forceinline__ float hi(uint32_t u) { return bf16_hi(u); }
+  static __device__ __forceinline__ uint32_t pack(float a, float b) { return pack_bf16(a, b); }
+};
+template <> struct Pk<_Float16> {
+  static __device__ __forceinline__ float lo(uint32_t u) { return (float)__builtin_bit_cast(f16x2_t, u).x; }
+  static __device__ __forceinline__ float hi(uint32_t u) { return (float)__builtin_bit_cast(f16x2_t, u).y; }
+  static __device__ __forceinline__ uint32_t pack(float a, float b) {
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+  }
+};
+
+template <typename E>
+__device__ __forceinline__ void unpack8e(const uint4& v, float (&f)[8]) {
+  f[0] = Pk<E>::lo(v.x); f[1] = Pk<E>::hi(v.x);
+  f[2] = Pk<E>::lo(v.y); f[3] = Pk<E>::hi(v.y);
+  f[4] = Pk<E>::lo(v.z); f[5] = Pk<E>::hi(v.z);
+  f[6] = Pk<E>::lo(v.w); f[7] = Pk<E>::hi(v.w);
+}
+
+template <typename E>
+__device__ __forceinline__ void add8e(const uint4& v, float (&f)[8]) {
+  f[0] += Pk<E>::lo(v.x); f[1] += Pk<E>::hi(v.x);
+  f[2] += Pk<E>::lo(v.y); f[3] += Pk<E>::hi(v.y);
+  f[4] += Pk<E>::lo(v.z); f[5] += Pk<E>::hi(v.z);
+  f[6] += Pk<E>::lo(v.w); f[7] += Pk<E>::hi(v.w);
+}
+
 // ---------------------------------------------------------------------------
 // Sums with a fixed association order.
 //
@@ -260,7 +295,7 @@ __device__ __forceinline__ void store16(__amdgpu_buffer_rsrc_t d, uint32_t off, 
 }
 
 // ---------------------------------------------------------------------------
-// Vector kernel, bf16.
+// Vector kernel, 16-bit element types (bf16; fp16 for the P = 1 ops).
 //   NP       number of partial buffers known at compile time, 0 = use np_rt
 //   VPT      16-byte vectors per lane per buffer; lane t owns vectors
 //            t, t + blockDim, ... (row length <= VPT * blockDim * 8 elements)
@@ -272,14 +307,14 @@ __device__ __forceinline__ void store16(__amdgpu_buffer_rsrc_t d, uint32_t off, 
 // ---------------------------------------------------------------------------
 //   Q        output kind (kQNone .. kQDynInt8); quant_scale is the static scale
 //            (kQStaticFp8) or the optional upper bound of the row scale (kQDynFp8)
-template <int NP, int VPT, int MAXNT, bool HAS_RES, bool COPY, int Q>
-__global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
-    PartialPtrs parts, int np_rt, void* y_out, void* residual, void* copy_out,
+//   E        element type of every tensor (__bf16 or _Float16)
+template <typename E, int NP, int VPT, int MAXNT, bool HAS_RES, bool COPY, int Q>
+__device__ __forceinline__ void row_norm_vec_body(
+    const PartialPtrs& parts, int np_rt, void* y_out, void* residual, void* copy_out,
     const void* __restrict__ weight, const float* __restrict__ quant_scale,
-    float* __restrict__ row_scales, float eps, int num_tokens, int vec_per_row, float hidden) {
+    float* __restrict__ row_scales, float eps, int num_tokens, int vec_per_row, float hidden,
+    float (*slots)[kMaxChunks], float (*max_slots)[16]) {
   constexpr bool FP8 = Q == kQStaticFp8;
-  __shared__ float slots[2][kMaxChunks];
-  __shared__ float max_slots[2][16];
   const int nt = blockDim.x;
   const int nwaves = nt >> 6;
   const int nchunks = (vec_per_row + 63) >> 6;  // <= VPT * nwaves
@@ -320,10 +355,10 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
         first[k] = a[k][0];
-        unpack8(a[k][0], s[k]);
+        unpack8e<E>(a[k][0], s[k]);
 #pragma unroll
-        for (int p = 1; p < NP; ++p) add8(a[k][p], s[k]);
-        if (HAS_RES) add8(rv[k], s[k]);
+        for (int p = 1; p < NP; ++p) add8e<E>(a[k][p], s[k]);
+        if (HAS_RES) add8e<E>(rv[k], s[k]);
       }
     } else {
       {
@@ -331,17 +366,17 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
 #pragma unroll
         for (int k = 0; k < VPT; ++k) {
           first[k] = load16<kLoadStream>(dp, off[k]);
-          unpack8(first[k], s[k]);
+          unpack8e<E>(first[k], s[k]);
         }
       }
       for (int p = 1; p < np; ++p) {
         const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[p], row, row_bytes);
 #pragma unroll
-        for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dp, off[k]), s[k]);
+        for (int k = 0; k < VPT; ++k) add8e<E>(load16<kLoadStream>(dp, off[k]), s[k]);
       }
       if (HAS_RES) {
 #pragma unroll
-        for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dr, off[k]), s[k]);
+        for (int k = 0; k < VPT; ++k) add8e<E>(load16<kLoadStream>(dr, off[k]), s[k]);
       }
     }
     // The weight row is fetched per token row, behind the row's own loads: it is
@@ -366,10 +401,10 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
       ss[k] = 0.0f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) ss[k] += s[k][e] * s[k][e];
-      rnew[k].x = pack_bf16(s[k][0], s[k][1]);
-      rnew[k].y = pack_bf16(s[k][2], s[k][3]);
-      rnew[k].z = pack_bf16(s[k][4], s[k][5]);
-      rnew[k].w = pack_bf16(s[k][6], s[k][7]);
+      rnew[k].x = Pk<E>::pack(s[k][0], s[k][1]);
+      rnew[k].y = Pk<E>::pack(s[k][2], s[k][3]);
+      rnew[k].z = Pk<E>::pack(s[k][4], s[k][5]);
+      rnew[k].w = Pk<E>::pack(s[k][6], s[k][7]);
       if (HAS_RES) store16(dr, off[k], rnew[k]);
     }
 
@@ -385,18 +420,18 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
         float w[8], t[8];
-        unpack8(wv[k], w);
+        unpack8e<E>(wv[k], w);
         uint4 tv;
-        tv.x = pack_bf16(s[k][0] * inv, s[k][1] * inv);
-        tv.y = pack_bf16(s[k][2] * inv, s[k][3] * inv);
-        tv.z = pack_bf16(s[k][4] * inv, s[k][5] * inv);
-        tv.w = pack_bf16(s[k][6] * inv, s[k][7] * inv);
-        unpack8(tv, t);
-        nv[k].x = pack_bf16(t[0] * w[0], t[1] * w[1]);
-        nv[k].y = pack_bf16(t[2] * w[2], t[3] * w[3]);
-        nv[k].z = pack_bf16(t[4] * w[4], t[5] * w[5]);
-        nv[k].w = pack_bf16(t[6] * w[6], t[7] * w[7]);
-        unpack8(nv[k], t);
+        tv.x = Pk<E>::pack(s[k][0] * inv, s[k][1] * inv);
+        tv.y = Pk<E>::pack(s[k][2] * inv, s[k][3] * inv);
+        tv.z = Pk<E>::pack(s[k][4] * inv, s[k][5] * inv);
+        tv.w = Pk<E>::pack(s[k][6] * inv, s[k][7] * inv);
+        unpack8e<E>(tv, t);
+        nv[k].x = Pk<E>::pack(t[0] * w[0], t[1] * w[1]);
+        nv[k].y = Pk<E>::pack(t[2] * w[2], t[3] * w[3]);
+        nv[k].z = Pk<E>::pack(t[4] * w[4], t[5] * w[5]);
+        nv[k].w = Pk<E>::pack(t[6] * w[6], t[7] * w[7]);
+        unpack8e<E>(nv[k], t);
 #pragma unroll
         for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(t[e]));
       }
@@ -407,7 +442,7 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
         float n[8];
-        unpack8(nv[k], n);
+        unpack8e<E>(nv[k], n);
         if (Q == kQDynInt8)
           store8(dy, off[k] / 2, quant4_int8(n[0], n[1], n[2], n[3], sinv),
                  quant4_int8(n[4], n[5], n[6], n[7], sinv));
@@ -421,16 +456,16 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       float r[8], w[8];
-      unpack8(rnew[k], r);
-      unpack8(wv[k], w);
+      unpack8e<E>(rnew[k], r);
+      unpack8e<E>(wv[k], w);
       uint4 o;
-      o.x = pack_bf16(r[0] * inv * w[0], r[1] * inv * w[1]);
-      o.y = pack_bf16(r[2] * inv * w[2], r[3] * inv * w[3]);
-      o.z = pack_bf16(r[4] * inv * w[4], r[5] * inv * w[5]);
-      o.w = pack_bf16(r[6] * inv * w[6], r[7] * inv * w[7]);
+      o.x = Pk<E>::pack(r[0] * inv * w[0], r[1] * inv * w[1]);
+      o.y = Pk<E>::pack(r[2] * inv * w[2], r[3] * inv * w[3]);
+      o.z = Pk<E>::pack(r[4] * inv * w[4], r[5] * inv * w[5]);
+      o.w = Pk<E>::pack(r[6] * inv * w[6], r[7] * inv * w[7]);
       if (FP8) {
         float y[8];
-        unpack8(o, y);
+        unpack8e<E>(o, y);
         store8(dy, off[k] / 2, quant4_fp8(y[0], y[1], y[2], y[3], scale_inv),
                quant4_fp8(y[4], y[5], y[6], y[7], scale_inv));
       } else {
@@ -438,6 +473,31 @@ __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
       }
     }
   }
+}
+
+template <int NP, int VPT, int MAXNT, bool HAS_RES, bool COPY, int Q>
+__global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
+    PartialPtrs parts, int np_rt, void* y_out, void* residual, void* copy_out,
+    const void* __restrict__ weight, const float* __restrict__ quant_scale,
+    float* __restrict__ row_scales, float eps, int num_tokens, int vec_per_row, float hidden) {
+  __shared__ float slots[2][kMaxChunks];
+  __shared__ float max_slots[2][16];
+  row_norm_vec_body<__bf16, NP, VPT, MAXNT, HAS_RES, COPY, Q>(parts, np_rt, y_out, residual, copy_out, weight,
+                                                            quant_scale, row_scales, eps, num_tokens,
+                                                            vec_per_row, hidden, slots, max_slots);
+}
+
+// fp16 tensors reach the library through the P = 1 ops only.
+template <int VPT, int MAXNT, bool HAS_RES, bool COPY, int Q>
+__global__ __launch_bounds__(MAXNT) void row_norm_f16_kernel(
+    PartialPtrs parts, void* y_out, void* residual, void* copy_out, const void* __restrict__ weight,
+    const float* __restrict__ quant_scale, float* __restrict__ row_scales, float eps, int num_tokens,
+    int vec_per_row, float hidden) {
+  __shared__ float slots[2][kMaxChunks];
+  __shared__ float max_slots[2][16];
+  row_norm_vec_body<_Float16, 1, VPT, MAXNT, HAS_RES, COPY, Q>(parts, 1, y_out, residual, copy_out, weight,
+                                                             quant_scale, row_scales, eps, num_tokens,
+                                                             vec_per_row, hidden, slots, max_slots);
 }
 
 // ---------------------------------------------------------------------------
@@ -611,6 +671,7 @@ struct RowNormArgs {
   void* residual;
   void* copy_out;
   const void* weight;
+  bool f16;                  // tensors are fp16 (vector kernel, P = 1 only); bf16 otherwise
   int q;                     // output kind (kQNone ..)
   const float* quant_scale;  // static fp8: the scale; dynamic fp8: optional upper bound (may be null)
   float* row_scales;         // dynamic kinds: one scale per row (output)
@@ -626,6 +687,19 @@ static int launch_vec(const RowNormArgs& a) {
   VecShape sh;
   if (!vec_shape(V, a.T, &sh)) return 1;  // caller falls back to the element-wise kernel
   dim3 g(a.grid), b(sh.nt);
+  if (a.f16) {
+    if (NP != 1) return 1;
+#define TW_LAUNCH_F16(VPT, MAXNT)                                                                \
+  hipLaunchKernelGGL((row_norm_f16_kernel<VPT, MAXNT, HAS_RES, COPY, Q>), g, b, 0, a.stream,     \
+                     a.parts, a.y, a.residual, a.copy_out, a.weight, a.quant_scale,              \
+                     a.row_scales, a.eps, (int)a.T, V, (float)a.H)
+    if (sh.vpt == 1) TW_LAUNCH_F16(1, 1024);
+    else if (sh.vpt == 2) TW_LAUNCH_F16(2, 1024);
+    else if (sh.maxnt == 256) TW_LAUNCH_F16(4, 256);
+    else TW_LAUNCH_F16(4, 1024);
+#undef TW_LAUNCH_F16
+    return 0;
+  }
 #define TW_LAUNCH(VPT, MAXNT)                                                                    \
   hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, MAXNT, HAS_RES, COPY, Q>), g, b, 0,          \
                      a.stream, a.parts, a.np, a.y, a.residual, a.copy_out, a.weight,             \
@@ -750,6 +824,7 @@ int run_row_norm_q(const char* what, const void* const* partials, int np, void* 
   a.residual = residual;
   a.copy_out = copy_out;
   a.weight = weight;
+  a.f16 = dtype == TW_DTYPE_F16;
   a.q = quant;
   a.quant_scale = quant_scale;
   a.row_scales = row_scales;
@@ -759,7 +834,7 @@ int run_row_norm_q(const char* what, const void* const* partials, int np, void* 
   a.grid = grid;
   a.stream = static_cast<hipStream_t>(stream_v);
 
-  if (vec_ok && dtype == TW_DTYPE_BF16) {
+  if (vec_ok && (dtype == TW_DTYPE_BF16 || (dtype == TW_DTYPE_F16 && np == 1))) {
     int fell = 1;
     switch (np) {
       case 1: fell = launch_vec_mode<1>(a); break;

@@ -67,59 +67,54 @@ def parse_args():
 
 
 class NormRunner:
-    """Pre-binds the C-ABI call for each input set so the timed loop is one ctypes
-    call per step (argument checks were done once, here, by the regular shim)."""
+    """One bound call (tokenweave_amd.ops.BoundOp: arguments checked once, a single
+    ctypes call per launch) for each input set, so that the host enqueues a step
+    faster than the GPU runs it."""
 
     def __init__(self, cfg, nsets, max_ctas, device, epilogue="bf16"):
         import torch
         from tokenweave_amd import _custom_ops as ops
         from tokenweave_amd import _lib
         from tokenweave_amd import workloads as wl
-        self.cfg, self.torch, self.lib = cfg, torch, _lib.lib()
-        self.sets, self.calls = [], []
+        self.calls = []
+        L = _lib.lib()
         for i in range(nsets):
             inp = wl.make_norm_inputs(cfg, device, seed_offset=i)
-            out = inp.partials[0]  # y lands on this rank's staging rows (rank 0)
-            # one checked call through the public shim validates the arguments
-            ops.reduce_add_rms_norm(inp.partials, out, inp.residual, inp.weight, cfg.eps,
-                                    max_ctas or None)
-            ptrs = (ctypes.c_void_p * cfg.P)(*[p.data_ptr() for p in inp.partials])
-            self.sets.append((inp, ptrs))
-            self.calls.append((ptrs, cfg.P, out.data_ptr(), inp.residual.data_ptr(),
-                               inp.weight.data_ptr(), cfg.T, cfg.H, max_ctas, cfg.eps))
-            if epilogue != "bf16":
-                self._bind_quant(i, epilogue, inp, ptrs, max_ctas, device)
+            if epilogue == "bf16":
+                # y lands on this rank's staging rows (rank 0)
+                op = ops.bind_reduce_add_rms_norm(inp.partials, inp.partials[0], inp.residual, inp.weight,
+                                                  cfg.eps, max_ctas or None)
+            else:
+                op = self._bind_quant(ops, L, torch, cfg, epilogue, inp, max_ctas, device)
+            op()  # one launch up front: a bad argument fails here, not in the timed loop
+            self.calls.append(op)
         torch.cuda.synchronize()
-        self.fn = {"bf16": self.lib.tw_reduce_add_rms_norm,
-                   "fp8_static": self.lib.tw_reduce_add_rms_norm_static_fp8_quant,
-                   "fp8_dynamic": self.lib.tw_reduce_add_rms_norm_dynamic_per_token_quant,
-                   "int8_dynamic": self.lib.tw_reduce_add_rms_norm_dynamic_per_token_quant}[epilogue]
 
-    def _bind_quant(self, i, epilogue, inp, ptrs, max_ctas, device):
-        """Replaces call i by the same reduction with a quantised output (one byte per
-        element into its own buffer, a float per row for the dynamic kinds)."""
-        torch, cfg = self.torch, self.cfg
-        from tokenweave_amd import _custom_ops as ops
+    @staticmethod
+    def _bind_quant(ops, L, torch, cfg, epilogue, inp, max_ctas, device):
+        """The same reduction with a quantised output (one byte per element into its own
+        buffer, a float per row for the dynamic kinds).  Checked once through the
+        regular shim, then frozen."""
         qdtype = torch.int8 if epilogue == "int8_dynamic" else torch.float8_e4m3fn
         out = torch.empty(cfg.T, cfg.H, dtype=qdtype, device=device)
         scales = torch.full((max(cfg.T, 1), 1), 0.05, dtype=torch.float32, device=device)
-        self.sets[i] = self.sets[i] + (out, scales)
+        ptrs = (ctypes.c_void_p * cfg.P)(*[p.data_ptr() for p in inp.partials])
+        keep = (inp, out, scales, ptrs)
         if epilogue == "fp8_static":
             ops.reduce_add_rms_norm_static_fp8_quant(inp.partials, out, inp.residual, inp.weight,
                                                      scales[:1].reshape(1), cfg.eps, max_ctas or None)
-            self.calls[i] = (ptrs, cfg.P, out.data_ptr(), inp.residual.data_ptr(), inp.weight.data_ptr(),
-                             scales.data_ptr(), cfg.T, cfg.H, max_ctas, cfg.eps)
-        else:
-            ops.reduce_add_rms_norm_dynamic_per_token_quant(inp.partials, out, scales, inp.residual,
-                                                            inp.weight, cfg.eps, None, max_ctas or None)
-            self.calls[i] = (ptrs, cfg.P, out.data_ptr(), scales.data_ptr(), inp.residual.data_ptr(),
-                             inp.weight.data_ptr(), None, cfg.T, cfg.H, max_ctas, cfg.eps,
-                             1 if epilogue == "int8_dynamic" else 0)
+            args = (ptrs, cfg.P, out.data_ptr(), inp.residual.data_ptr(), inp.weight.data_ptr(),
+                    scales.data_ptr(), cfg.T, cfg.H, max_ctas, cfg.eps)
+            return ops.BoundOp(L.tw_reduce_add_rms_norm_static_fp8_quant, args, keep, out.device)
+        ops.reduce_add_rms_norm_dynamic_per_token_quant(inp.partials, out, scales, inp.residual,
+                                                        inp.weight, cfg.eps, None, max_ctas or None)
+        args = (ptrs, cfg.P, out.data_ptr(), scales.data_ptr(), inp.residual.data_ptr(),
+                inp.weight.data_ptr(), None, cfg.T, cfg.H, max_ctas, cfg.eps,
+                1 if epilogue == "int8_dynamic" else 0)
+        return ops.BoundOp(L.tw_reduce_add_rms_norm_dynamic_per_token_quant, args, keep, out.device)
 
-    def step(self, i, stream_ptr):
-        rc = self.fn(*self.calls[i % len(self.calls)], stream_ptr)
-        if rc != 0:
-            raise RuntimeError(self.lib.tw_last_error().decode())
+    def step(self, i, stream):
+        self.calls[i % len(self.calls)](stream)
 
 
 def quant_bytes(cfg, epilogue):
@@ -139,9 +134,8 @@ def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16"):
     nsets = max(2, min(nsets, int(free * 0.6) // (set_bytes * 3)))  # fp32 staging while generating
     runner = NormRunner(cfg, nsets, max_ctas, device, epilogue)
     stream = torch.cuda.current_stream()
-    sp = ctypes.c_void_p(stream.cuda_stream)
     for i in range(warmup):
-        runner.step(i, sp)
+        runner.step(i, stream)
     torch.cuda.synchronize()
     # timed region: exactly `steps` launches between two synchronisation points,
     # bracketed by HIP events on the launch stream
@@ -149,7 +143,7 @@ def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16"):
     t0 = time.perf_counter()
     e0.record(stream)
     for i in range(steps):
-        runner.step(i, sp)
+        runner.step(i, stream)
     e1.record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -184,13 +178,12 @@ def time_norm_warm(cfg, steps, max_ctas, device):
     import torch
     runner = NormRunner(cfg, 1, max_ctas, device)
     stream = torch.cuda.current_stream()
-    sp = ctypes.c_void_p(stream.cuda_stream)
     for i in range(10):
-        runner.step(0, sp)
+        runner.step(0, stream)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
     for i in range(steps):
-        runner.step(0, sp)
+        runner.step(0, stream)
     e1.record(stream)
     torch.cuda.synchronize()
     del runner
@@ -236,32 +229,27 @@ def time_weave(device, norm_cap, gemm_cap, steps=200):
     a stage faster than the GPU runs it."""
     import torch
     from tokenweave_amd import _custom_ops as ops
-    from tokenweave_amd import _lib
     from tokenweave_amd import workloads as wl
     cfg, R = wl.C5_NORM, 8
-    L = _lib.lib()
     inps = [wl.make_norm_inputs(cfg, device, seed_offset=i) for i in range(R)]
     g = wl.make_gemm_inputs(device=device)
     Ta, K = g.a.shape
     N = g.b.shape[0]
     stages = [torch.zeros((Ta, N), dtype=torch.bfloat16, device=device) for _ in range(R)]
-    for i in range(R):  # validate once through the shims
-        ops.gemm_bf16_nt(stages[i], g.a, g.b, max_cus=gemm_cap or None)
-        ops.reduce_add_rms_norm(inps[i].partials, inps[i].partials[0], inps[i].residual,
-                                inps[i].weight, cfg.eps, norm_cap or None)
-    ptrs = [(ctypes.c_void_p * cfg.P)(*[p.data_ptr() for p in inp.partials]) for inp in inps]
     main_s, side_s = torch.cuda.Stream(), torch.cuda.Stream()
-    pm, ps = ctypes.c_void_p(main_s.cuda_stream), ctypes.c_void_p(side_s.cuda_stream)
+    gemms, norms = {}, {}
+    for cap in {0, gemm_cap}:
+        gemms[cap] = [ops.bind_gemm_bf16_nt(stages[i], g.a, g.b, cap or None) for i in range(R)]
+    for cap in {0, norm_cap}:
+        norms[cap] = [ops.bind_reduce_add_rms_norm(inp.partials, inp.partials[0], inp.residual, inp.weight,
+                                                   cfg.eps, cap or None) for inp in inps]
+    pm, ps = main_s, side_s
 
-    def gemm(i, cap, sp):
-        rc = L.tw_gemm_bf16_nt(stages[i % R].data_ptr(), g.a.data_ptr(), g.b.data_ptr(), Ta, N, K, N, cap, sp)
-        assert rc == 0, _lib.last_error()
+    def gemm(i, cap, stream):
+        gemms[cap][i % R](stream)
 
-    def norm(i, cap, sp):
-        inp = inps[i % R]
-        rc = L.tw_reduce_add_rms_norm(ptrs[i % R], cfg.P, inp.partials[0].data_ptr(), inp.residual.data_ptr(),
-                                      inp.weight.data_ptr(), cfg.T, cfg.H, cap, cfg.eps, sp)
-        assert rc == 0, _lib.last_error()
+    def norm(i, cap, stream):
+        norms[cap][i % R](stream)
 
     def weave(i):
         before = torch.cuda.Event()

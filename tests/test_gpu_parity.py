@@ -421,3 +421,32 @@ def test_empty_batch_is_a_no_op():
     ops.fused_add_rms_norm(x, x.clone(), w, 1e-5)
     ops.reduce_add_rms_norm([x, x.clone()], x.clone(), x.clone(), w, 1e-5)
     torch.cuda.synchronize()
+
+
+def test_bound_ops_equal_the_regular_ops_and_follow_the_given_stream():
+    """BoundOp: arguments checked at bind time, one C call per launch afterwards."""
+    cfg = wl.C2.with_tokens(48)
+    inp = wl.make_norm_inputs(cfg, DEV)
+    y_ref, r_ref = torch.empty_like(inp.residual), inp.residual.clone()
+    ops.reduce_add_rms_norm(inp.partials, y_ref, r_ref, inp.weight, cfg.eps)
+    y, r = torch.empty_like(inp.residual), inp.residual.clone()
+    op = ops.bind_reduce_add_rms_norm(inp.partials, y, r, inp.weight, cfg.eps, MAX_CTAS=5)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    op(side)
+    side.synchronize()
+    assert torch.equal(y, y_ref) and torch.equal(r, r_ref)
+    r.copy_(inp.residual)
+    y.zero_()
+    op()                       # current stream
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_ref) and torch.equal(r, r_ref)
+    g = wl.make_gemm_inputs(200, 256, 128, DEV, seed=3)
+    out_ref = torch.empty(200, 256, dtype=torch.bfloat16, device=DEV)
+    out = torch.empty_like(out_ref)
+    ops.gemm_bf16_nt(out_ref, g.a, g.b)
+    ops.bind_gemm_bf16_nt(out, g.a, g.b)()
+    torch.cuda.synchronize()
+    assert torch.equal(out, out_ref)
+    with pytest.raises(RuntimeError, match="same shape"):
+        ops.bind_reduce_add_rms_norm(inp.partials, y[:10], r, inp.weight, cfg.eps)

@@ -174,3 +174,13 @@ def test_weave_config_table_and_plan():
     table = {1024: {"attention_ctas": 8, "mlp_ctas": 4, "split_offset": 256}}
     assert tw.weave_plan(1100, table) == {"split_size": 896, "rest_size": 204, "attention_ctas": 8,
                                           "mlp_ctas": 4, "gemm_cus": 0}
+
+
+def test_bind_checks_arguments_at_bind_time():
+    import tokenweave_amd._custom_ops as ops
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    w = torch.ones(64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.bind_reduce_add_rms_norm([x], x, x.clone(), w, 1e-5)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.bind_gemm_bf16_nt(torch.zeros(4, 4, dtype=torch.bfloat16), x, x)

@@ -236,11 +236,32 @@ def fused_rs_ln_cta(input: torch.Tensor, residual: torch.Tensor, weight: torch.T
 # ---------------------------------------------------------------------------
 # one-GPU general form and the weave GEMM (no counterpart in vllm/_custom_ops.py)
 # ---------------------------------------------------------------------------
-def reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
-                        residual: torch.Tensor, weight: torch.Tensor, epsilon: float,
-                        MAX_CTAS: Optional[int] = None) -> None:
-    """out <- RMSNorm(sum_p partials[p] + residual) * weight; residual <- the sum.
-    `out` may be one of the partials."""
+class BoundOp:
+    """An op whose arguments were checked once and frozen into one C-ABI call.
+
+    `op()` enqueues it on the current stream of the tensors' device, `op(stream)` on
+    the given `torch.cuda.Stream`: a single ctypes call, for loops where the regular
+    shims' argument checks (several microseconds of Python) would outlast the kernel.
+    The bound tensors are kept alive; their addresses and shapes must not change."""
+    __slots__ = ("_fn", "_args", "_keep", "_device", "_index")
+
+    def __init__(self, fn, args, keep, device):
+        self._fn, self._args, self._keep, self._device = fn, args, keep, device
+        self._index = device.index if device.index is not None else torch.cuda.current_device()
+
+    def __call__(self, stream: Optional[torch.cuda.Stream] = None) -> None:
+        if stream is None:
+            stream = torch.cuda.current_stream(self._device)
+        if torch.cuda.current_device() != self._index:
+            with torch.cuda.device(self._index):
+                rc = self._fn(*self._args, stream.cuda_stream)
+        else:
+            rc = self._fn(*self._args, stream.cuda_stream)
+        if rc:
+            _lib.check(rc)
+
+
+def _prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS):
     P = len(partials)
     _require(1 <= P <= _lib.TW_MAX_PARTIALS,
              f"number of partials {P} not in [1, {_lib.TW_MAX_PARTIALS}]")
@@ -255,10 +276,23 @@ def reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
         _require(p.shape == out.shape, f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(out.shape)}")
     _check_weight(weight, H, torch.bfloat16, dev)
     ptrs = (ctypes.c_void_p * P)(*[p.data_ptr() for p in partials])
-    with _on_device(out):
-        _lib.check(_lib.lib().tw_reduce_add_rms_norm(
-            ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H,
-            _cap(MAX_CTAS), epsilon, _stream_ptr(out)))
+    args = (ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H, _cap(MAX_CTAS), epsilon)
+    return _lib.lib().tw_reduce_add_rms_norm, args, (list(partials), out, residual, weight), dev
+
+
+def reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
+                        residual: torch.Tensor, weight: torch.Tensor, epsilon: float,
+                        MAX_CTAS: Optional[int] = None) -> None:
+    """out <- RMSNorm(sum_p partials[p] + residual) * weight; residual <- the sum.
+    `out` may be one of the partials."""
+    BoundOp(*_prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS))()
+
+
+def bind_reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
+                             residual: torch.Tensor, weight: torch.Tensor, epsilon: float,
+                             MAX_CTAS: Optional[int] = None) -> BoundOp:
+    """`reduce_add_rms_norm` with the checks done now and the launch deferred."""
+    return BoundOp(*_prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS))
 
 
 # ---------------------------------------------------------------------------
@@ -428,11 +462,7 @@ def reduce_add_rms_norm_dynamic_per_token_quant(partials: Sequence[torch.Tensor]
             _stream_ptr(first)))
 
 
-def gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
-                 max_cus: Optional[int] = None) -> None:
-    """out[M, N] <- a[M, K] @ b[N, K]^T (bf16, fp32 accumulate).  `out` may be a row
-    slice of a wider buffer (row stride >= N).  The in-place row-parallel linear of
-    vllm/model_executor/layers/linear.py:203-228."""
+def _prepare_gemm_bf16_nt(out, a, b, max_cus):
     _require_bf16("gemm_bf16_nt_kernel", a)
     dev = a.device
     _check_tensor("a", a, torch.bfloat16, dev)
@@ -446,9 +476,22 @@ def gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
     _require(tuple(out.shape) == (M, N), f"out has shape {tuple(out.shape)}, expected {(M, N)}")
     _require(out.stride(1) == 1 and (M <= 1 or out.stride(0) >= N), "out rows must be contiguous")
     ldc = out.stride(0) if M > 1 else max(N, out.stride(0))
-    with _on_device(a):
-        _lib.check(_lib.lib().tw_gemm_bf16_nt(out.data_ptr(), a.data_ptr(), b.data_ptr(), M, N, K,
-                                              ldc, _cap(max_cus), _stream_ptr(a)))
+    args = (out.data_ptr(), a.data_ptr(), b.data_ptr(), M, N, K, ldc, _cap(max_cus))
+    return _lib.lib().tw_gemm_bf16_nt, args, (out, a, b), dev
+
+
+def gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
+                 max_cus: Optional[int] = None) -> None:
+    """out[M, N] <- a[M, K] @ b[N, K]^T (bf16, fp32 accumulate).  `out` may be a row
+    slice of a wider buffer (row stride >= N).  The in-place row-parallel linear of
+    vllm/model_executor/layers/linear.py:203-228."""
+    BoundOp(*_prepare_gemm_bf16_nt(out, a, b, max_cus))()
+
+
+def bind_gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
+                      max_cus: Optional[int] = None) -> BoundOp:
+    """`gemm_bf16_nt` with the checks done now and the launch deferred."""
+    return BoundOp(*_prepare_gemm_bf16_nt(out, a, b, max_cus))
 
 
 def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:

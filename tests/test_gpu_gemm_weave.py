@@ -77,6 +77,9 @@ def test_gemm_output_with_wide_row_stride():
     (300, 384, 128, 388, 0),    # row stride % 8 != 0: 8-byte stores
     (300, 384, 128, 384, 4),    # out 8-byte but not 16-byte aligned: 8-byte stores
     (645, 520, 192, 520, 0),    # ragged tile edges in both directions, 16-byte stores
+    (2048, 10240, 128, 10240, 0),   # 8 x 27 tiles of 256 x 384 fit one round of 256 compute units
+    (2000, 10004, 128, 10004, 0),   # the same tile with ragged edges and 8-byte stores
+    (2040, 10000, 192, 10008, 0),   # ... and with 16-byte stores into a wider buffer
 ])
 def test_gemm_large_tile_kernel_store_paths(M, N, K, ldc, shift):
     print(f"[case] gemm stores M={M} N={N} K={K} ldc={ldc} shift={shift}", flush=True)

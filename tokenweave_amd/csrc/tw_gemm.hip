@@ -12,12 +12,12 @@
 // whole 128-byte lines per row.
 //
 // Two kernels:
-//  * gemm_bf16_nt_big_kernel<TM> (K % 64 == 0): (64 TM) x 256 x 64 tiles, TM = 3,
-//    4 or 5 chosen per problem so that the tile count wastes the fewest workgroup
-//    rounds (M = 2458: 320-row tiles make exactly 256 tiles), 8 waves (2 x 4, two
-//    per SIMD), each wave (32 TM) x 64 (up to 160 fp32 accumulators).  Operand
-//    slabs go from global memory straight into LDS (buffer_load ... lds: no
-//    staging registers, no LDS store instructions), two LDS stages of 56-72 KiB.
+//  * gemm_bf16_nt_big_kernel<TM, TN> (K % 64 == 0): (64 TM) x (128 TN) x 64 tiles,
+//    8 waves (2 x 4, two per SIMD), each wave (32 TM) x (32 TN): 192/256/320 x 256
+//    (TN = 2) chosen per problem so that the tile count wastes the fewest workgroup
+//    rounds (M = 2458: 320-row tiles make exactly 256 tiles), or 256 x 384.
+//    Operand slabs go from global memory straight into LDS (buffer_load ... lds:
+//    no staging registers, no LDS store instructions), two LDS stages.
 //    A wave instruction fills 1 KiB = 8 LDS rows of 128 bytes; row r keeps its
 //    16-byte chunk c at position c ^ ((r >> 1) & 7), which makes the 16-byte
 //    fragment reads of 16 consecutive rows conflict-free on the 64-bank LDS
@@ -288,6 +288,56 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
                                (uint32_t)(kt + 1) * BIG_ROWB);
       const uint8_t* pa = lds_big + stage * STAGE + (wm * WM) * BIG_ROWB;
       const uint8_t* pb = lds_big + stage * STAGE + PANEL_A + (wn * WN) * BIG_ROWB;
+      if constexpr (TN == 3) {
+        // 192 accumulators leave no room for two copies of both fragment sets: `a`
+        // fragments are single-buffered and refilled for the next step right after
+        // their last use in this one (half of them in the middle of the step, half
+        // at its end); only the `b` fragments are double-buffered.
+        bf16x8_t fa[TM], fb[2][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          fa[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(pa + i * 32 * BIG_ROWB + roff[0]));
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          fb[0][j] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(pb + j * 32 * BIG_ROWB + roff[0]));
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const int cur = kk & 1, nxt = cur ^ 1;
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int i = 0; i < H1; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[i], acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (kk < 3) {
+#pragma unroll
+            for (int i = 0; i < H1; ++i)
+              fa[i] = __builtin_bit_cast(
+                  bf16x8_t, *reinterpret_cast<const uint4*>(pa + i * 32 * BIG_ROWB + roff[kk + 1]));
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+              fb[nxt][j] = __builtin_bit_cast(
+                  bf16x8_t, *reinterpret_cast<const uint4*>(pb + j * 32 * BIG_ROWB + roff[kk + 1]));
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int i = H1; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[i], acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (kk < 3) {
+#pragma unroll
+            for (int i = H1; i < TM; ++i)
+              fa[i] = __builtin_bit_cast(
+                  bf16x8_t, *reinterpret_cast<const uint4*>(pa + i * 32 * BIG_ROWB + roff[kk + 1]));
+          }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        continue;
+      }
       bf16x8_t fa[2][TM], fb[2][TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -341,10 +391,10 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
       // stages are free: every wave passed the barrier that ends the k loop.
       constexpr int PATCH_ROW = WN * 2 + 8;            // bytes
       constexpr int CHUNKS = WN / 8;                   // 16-byte chunks per patch row
-      constexpr int ROWS_PER_PASS = 64 / CHUNKS;
-      static_assert(64 % CHUNKS == 0 && 32 % ROWS_PER_PASS == 0, "patch read-back shape");
+      constexpr int ROWS_PER_PASS = 64 / CHUNKS;       // 8 (WN = 64) or 5 (WN = 96: 4 lanes idle)
       uint8_t* patch = lds_big + wave * (32 * PATCH_ROW);
       const int rd_row = lane / CHUNKS, rd_chunk = lane % CHUNKS;
+      const bool rd_lane = rd_row < ROWS_PER_PASS;
       const int n = n0 + wn * WN + rd_chunk * 8;
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
@@ -362,12 +412,12 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
         for (int r = 0; r < 32; r += ROWS_PER_PASS) {
-          const int row = r + rd_row;
+          const int row = min(r + rd_row, 31);
           const int m = m0 + wm * WM + i * 32 + row;
           // 8-byte LDS reads: the padded row pitch keeps rows 8-byte, not 16-byte, aligned
           const uint2 lo = *reinterpret_cast<const uint2*>(patch + row * PATCH_ROW + rd_chunk * 16);
           const uint2 hi = *reinterpret_cast<const uint2*>(patch + row * PATCH_ROW + rd_chunk * 16 + 8);
-          if (m < M && n < N)
+          if (rd_lane && r + rd_row < 32 && m < M && n < N)
             *reinterpret_cast<uint4*>(out + (size_t)m * ldc + n) = make_uint4(lo.x, lo.y, hi.x, hi.y);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -419,21 +469,25 @@ static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64
   return TW_OK;
 }
 
-// Workgroup tile for the problem, (64 TM) x (128 TN).  Cost = rounds x (tile area + a
-// fixed part per round); ties go to the smaller tile.  Only 64-wide wave tiles (TN = 2)
-// are offered: 96 x 96 wave tiles (192 x 384 workgroup tiles), which read a third
-// fewer LDS fragments per MFMA, measured no faster per tile and fit the compute-unit
-// count worse on the shapes of interest.
+// Workgroup tile for the problem, (64 TM) x (128 TN).  Cost = rounds x (tile area /
+// relative throughput + a fixed part per round); ties go to the earlier entry.  The
+// 64-wide wave tiles come in three heights so that a tile count can be made to fit the
+// compute units exactly (M = 2458: 320-row tiles make 256 tiles); 256 x 384 (96-wide
+// wave tiles, 192 accumulators, exactly 160 KiB of LDS) wins where its fewer, larger
+// rounds fit.  96 x 96 wave tiles (192 x 384) were measured no faster per area than
+// 256 x 256 and are not offered.
 struct BigTile { int tm, tn; };
 
 static BigTile pick_big_tile(int64_t M, int64_t N, int cus) {
-  static const struct { int tm, tn; } kTiles[] = {{3, 2}, {4, 2}, {5, 2}};
+  // Relative throughput per tile area, measured: the 256 x 384 tile loads a fifth fewer
+  // operand bytes per flop and runs a round in 1.35x the time of a 256 x 256 round.
+  static const struct { int tm, tn; double eff; } kTiles[] = {{3, 2, 1.0}, {4, 2, 1.0}, {5, 2, 1.0}, {4, 3, 1.1}};
   BigTile best = {4, 2};
   double best_cost = 1e300;
   for (const auto& t : kTiles) {
     const int64_t tiles = ((M + 64 * t.tm - 1) / (64 * t.tm)) * ((N + 128 * t.tn - 1) / (128 * t.tn));
     const int64_t rounds = (tiles + cus - 1) / cus;
-    const double cost = (double)rounds * (64.0 * t.tm * 128.0 * t.tn + 2048.0);
+    const double cost = (double)rounds * (64.0 * t.tm * 128.0 * t.tn / t.eff + 2048.0);
     if (cost < best_cost) {
       best_cost = cost;
       best = BigTile{t.tm, t.tn};
@@ -467,7 +521,8 @@ int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t
     const uint16_t* pb = static_cast<const uint16_t*>(b);
     int rc;
     const BigTile bt = pick_big_tile(M, N, cus);
-    if (bt.tm == 3) rc = launch_big<3, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
+    if (bt.tn == 3) rc = launch_big<4, 3>(o, pa, pb, M, N, K, ldc, max_cus, hs);
+    else if (bt.tm == 3) rc = launch_big<3, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
     else if (bt.tm == 5) rc = launch_big<5, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
     else rc = launch_big<4, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
     if (rc != TW_OK) return rc;

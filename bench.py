@@ -192,8 +192,9 @@ def time_norm_warm(cfg, steps, max_ctas, device):
 
 
 def cpu_baseline(cfg, budget_s):
-    """Times the CPU checker on a bounded sample of the workload: the same shapes,
-    rows capped so one call stays around a second, repeated inside the budget."""
+    """Times the CPU checker on a bounded sample of the workload: the same shapes (rows
+    capped at 1024), rotating through input sets of 1 GiB in total so that, like the GPU
+    legs, every call reads memory and not a cache, repeated for `budget_s` seconds."""
     import numpy as np
     import torch
     from oracle import tw_oracle as O
@@ -201,23 +202,27 @@ def cpu_baseline(cfg, budget_s):
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
     rows = min(cfg.T, 1024)
     sample = cfg.with_tokens(rows)
-    inp = wl.make_norm_inputs(sample, "cpu")
     bits = lambda t: np.ascontiguousarray(t.contiguous().view(torch.int16).numpy().view(np.uint16))
-    parts = [bits(p) for p in inp.partials]
-    r, w = bits(inp.residual), bits(inp.weight)
-    y = np.empty_like(r)
-    O.reduce_add_rms_norm(parts, r, w, cfg.eps, y=y)  # warm-up (page faults, thread pool)
+    nsets = max(2, min(32, -(-(1 << 30) // sample.bytes)))
+    sets = []
+    for i in range(nsets):
+        inp = wl.make_norm_inputs(sample, "cpu", seed_offset=i)
+        r = bits(inp.residual)
+        sets.append(([bits(p) for p in inp.partials], r, bits(inp.weight), np.empty_like(r)))
+    for parts, r, w, y in sets[:2]:   # warm-up (page faults, thread pool)
+        O.reduce_add_rms_norm(parts, r, w, cfg.eps, y=y)
     times, t_end = [], time.perf_counter() + budget_s
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 200):
+    while len(times) < 3 or time.perf_counter() < t_end:
+        parts, r, w, y = sets[len(times) % nsets]
         t0 = time.perf_counter()
         O.reduce_add_rms_norm(parts, r, w, cfg.eps, y=y)
         times.append(time.perf_counter() - t0)
     med = statistics.median(times)
     return {"value": round(sample.bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads,
             "kind": "port",
-            "sample": f"{len(times)} calls of P={sample.P} T={rows} H={sample.H} "
-                      f"({sample.bytes} algorithmic bytes each), median {med * 1e6:.0f} us/call, "
-                      f"OpenMP over rows with {threads} threads"}
+            "sample": f"{len(times)} calls in {budget_s:.0f} s of P={sample.P} T={rows} H={sample.H} "
+                      f"({sample.bytes} algorithmic bytes each) over {nsets} rotating input sets, "
+                      f"median {med * 1e6:.0f} us/call, OpenMP over rows with {threads} threads"}
 
 
 def time_weave(device, norm_cap, gemm_cap, steps=200):

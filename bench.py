@@ -352,6 +352,20 @@ def main():
                            "gbps": round(c.bytes / r["kernel_us_mean"] / 1e3, 1),
                            "pct_hbm_peak": round(c.bytes / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
             log(f"[sweep] {name}: {sweep[name]}")
+        # The reference's own microbenchmark grid for the P = 1 op (fused_add_rms_norm_cta,
+        # H = 8192; artifact/csvs/figure_4.csv, one H100): context, not a baseline for the
+        # headline metric, whose P = 8 form the reference does not publish.
+        for rows, h100_us in ((64, 8.61), (256, 12.16), (1024, 29.92), (2048, 51.84), (4096, 96.51),
+                              (32768, 712.4)):
+            c = wl.C1.with_tokens(rows, f"p1_add_rms_norm@T{rows}")
+            steps = max(50, min(2000, int(0.02 * 5e12 / c.bytes)))
+            r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device)
+            sweep[c.name] = {"P": 1, "T": rows, "H": c.H, "bytes": c.bytes,
+                             "kernel_us": round(r["kernel_us_mean"], 3),
+                             "gbps": round(c.bytes / r["kernel_us_mean"] / 1e3, 1),
+                             "pct_hbm_peak": round(c.bytes / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2),
+                             "reference_h100_us": h100_us}
+            log(f"[sweep] {c.name}: {sweep[c.name]}")
         for name in ("c2_llama70b_tp8_shard@T256", "c2_unsharded@T2048"):
             c = cfgs[name]
             steps = max(50, min(2000, int(0.02 * 5e12 / c.bytes)))

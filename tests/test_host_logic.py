@@ -184,3 +184,42 @@ def test_bind_checks_arguments_at_bind_time():
         ops.bind_reduce_add_rms_norm([x], x, x.clone(), w, 1e-5)
     with pytest.raises(RuntimeError, match="GPU only"):
         ops.bind_gemm_bf16_nt(torch.zeros(4, 4, dtype=torch.bfloat16), x, x)
+
+
+def test_fuse_only_schedule_calls_in_reference_order():
+    """tokenweave_with_fuse_only (reference tokenweave_utils.py:95-172): layer-0 norm with
+    out=residual, attention on the actual tokens, post-attention fused norm, MLP, fused
+    norm of the next layer — with the shard arithmetic of fused_allreduce_layernorm."""
+    log = []
+
+    class Norm:
+        def __init__(self, name):
+            self.name = name
+
+        def __call__(self, x, residual=None, out=None, **kw):
+            log.append((self.name, tuple(x.shape), "out" if out is not None else "res", kw.get("offset"),
+                        kw.get("MAX_CTAS"), kw.get("fused_ar", False)))
+
+    class Layer:
+        input_layernorm = Norm("input")
+        post_attention_layernorm = Norm("post")
+
+        def self_attn(self, positions, hidden_states):
+            log.append(("attn", tuple(hidden_states.shape)))
+
+    hs = torch.zeros(16, 8, dtype=torch.bfloat16)
+    res = torch.zeros_like(hs)
+    tw.tokenweave_with_fuse_only(Layer(), torch.arange(13), hs, res, object(), 0, rank=2, world_size=4,
+                                 next_layer_norm=Norm("next"), actual_tokens=13,
+                                 nearest_multiple_of_world_size=16, MAX_CTAS_ATTN=3, MAX_CTAS_MLP=32,
+                                 mlp_fn=lambda x: log.append(("mlp", tuple(x.shape))))
+    row_bytes = 8 * 2
+    assert log == [
+        ("input", (16, 8), "out", None, None, False),
+        ("attn", (13, 8)),
+        ("post", (4, 8), "res", 2 * 4 * row_bytes, 3, True),
+        ("mlp", (13, 8)),
+        ("next", (4, 8), "res", 2 * 4 * row_bytes, 4, True),   # MAX_CTAS is capped by the shard's rows
+    ]
+    with pytest.raises(AssertionError, match="mlp_fn"):
+        tw.tokenweave_with_fuse_only(Layer(), None, hs, res, object(), 1, nearest_multiple_of_world_size=16)

@@ -3,9 +3,11 @@ that stand in for symmetric memory on one GPU, and the two-stream weave step.
 
 Mirror of ``vllm/model_executor/models/tokenweave_utils.py``:
 ``fused_allreduce_layernorm`` (:24-92) keeps its argument list, assertions and
-slice/offset arithmetic; ``weave_norm_gemm`` is one stage of
-``tokenweave_overlap`` (:236-260) — the norm of one token split on a second
-stream while the other split's row-parallel GEMM runs on the current stream.
+slice/offset arithmetic; ``tokenweave_with_fuse_only`` (:95-172) and
+``tokenweave_overlap`` (:175-340) keep theirs and the order of their stream
+hand-offs; ``weave_norm_gemm`` is one stage of the overlap — the norm of one
+token split on a second stream while the other split's row-parallel GEMM runs
+on the current stream.
 """
 from __future__ import annotations
 
@@ -224,3 +226,153 @@ def weave_norm_gemm(gemm: Callable[[], None], norm: Callable[[], None],
         with torch.cuda.stream(norm_stream):
             norm()
     current.wait_stream(norm_stream)
+
+
+def _shard_rows(total_tokens: int, rank: int, world_size: int, all_ranks: bool):
+    """row_range for fused_allreduce_layernorm: None = the reference's even split
+    for `rank`; every row when one process plays all the ranks."""
+    return (0, total_tokens) if all_ranks else None
+
+
+def tokenweave_with_fuse_only(
+    self,
+    positions: torch.Tensor,
+    hidden_states: torch.Tensor,
+    residual: Optional[torch.Tensor],
+    symm_mem_hdl: Any,
+    layer_id: int,
+    rank: int = 0,
+    world_size: int = 1,
+    next_layer_norm: Optional[RMSNorm] = None,
+    actual_tokens: Optional[int] = None,
+    nearest_multiple_of_world_size: Optional[int] = None,
+    MAX_CTAS_ATTN: int = 16,
+    MAX_CTAS_MLP: int = 16,
+    mlp_fn: Optional[Callable] = None,
+    all_ranks: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One decoder layer with the fused reduce + add + norm after attention and
+    after the MLP, no overlap (reference tokenweave_utils.py:95-172, same
+    arguments).  `self` is the layer: it provides `input_layernorm`,
+    `post_attention_layernorm` and `self_attn(positions=, hidden_states=)`, whose
+    row-parallel output projection leaves this rank's partial sum in
+    `hidden_states` (this rank's staging rows); `mlp_fn` does the same for the MLP.
+
+    `all_ranks=True` (no counterpart in the reference) normalises every row instead
+    of this rank's shard: one GPU standing in for all the ranks, whose shards the
+    all-gather would have delivered."""
+    assert mlp_fn is not None, "mlp_fn must be provided"
+    num_tokens_per_rank = nearest_multiple_of_world_size // world_size
+    rows = _shard_rows(hidden_states.shape[0], rank, world_size, all_ranks)
+    if residual is None:
+        residual = torch.empty_like(hidden_states)
+    if layer_id == 0:
+        self.input_layernorm(hidden_states, out=residual)
+
+    self.self_attn(positions=positions, hidden_states=hidden_states[:actual_tokens])
+    fused_allreduce_layernorm(
+        layernorm=self.post_attention_layernorm, hidden_states=hidden_states, residual=residual,
+        symm_mem_hdl=symm_mem_hdl, num_tokens_per_rank=num_tokens_per_rank, rank=rank,
+        world_size=world_size, MAX_CTAS=MAX_CTAS_ATTN, row_range=rows)
+    mlp_fn(hidden_states[:actual_tokens])
+    fused_allreduce_layernorm(
+        layernorm=next_layer_norm, hidden_states=hidden_states, residual=residual,
+        symm_mem_hdl=symm_mem_hdl, num_tokens_per_rank=num_tokens_per_rank, rank=rank,
+        world_size=world_size, MAX_CTAS=MAX_CTAS_MLP, row_range=rows)
+    return hidden_states, residual
+
+
+def tokenweave_overlap(
+    self,
+    positions: torch.Tensor,
+    hidden_states: torch.Tensor,
+    residual: Optional[torch.Tensor],
+    symm_mem_hdl: Any,
+    layer_id: int,
+    end_layer: Optional[int] = None,
+    rank: int = 0,
+    world_size: int = 1,
+    current_stream: Optional[torch.cuda.Stream] = None,
+    copy_stream: Optional[torch.cuda.Stream] = None,
+    next_layer_norm: Optional[RMSNorm] = None,
+    split_size: Optional[int] = None,
+    actual_tokens: Optional[int] = None,
+    num_tokens_padded: Optional[int] = None,
+    MAX_CTAS_ATTN: int = 16,
+    MAX_CTAS_MLP: int = 16,
+    mlp_fn: Optional[Callable] = None,
+    all_ranks: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One decoder layer under the TokenWeave schedule (reference
+    tokenweave_utils.py:175-340, same arguments and the same order of hand-offs):
+    the tokens are cut at `split_size`; while one split computes (attention, MLP) on
+    `current_stream`, the fused reduce + add + norm of the other runs on
+    `copy_stream`.  Every compute step ends with `current_stream.wait_stream(copy_stream)`
+    and every norm starts with `copy_stream.wait_stream(current_stream)`, exactly as
+    in the reference, so the result equals the unsplit schedule's.
+
+    Layer 0 (reference :203-226): split 0 has nothing to reduce and takes
+    `input_layernorm(x, out=residual)`; for split 1 the reference reduce-scatters,
+    normalises its shard and all-gathers — on one GPU that is the fused op on a
+    zeroed residual (residual <- sum of the partials, x <- norm of it).
+    The last layer normalises split 1 after its MLP on the current stream (:327-339)."""
+    assert mlp_fn is not None, "mlp_fn must be provided"
+    hidden = hidden_states.shape[1]
+    offset_second = split_size * hidden * hidden_states.element_size()
+    if residual is None:
+        residual = torch.empty_like(hidden_states)
+    hidden_states_1, hidden_states_2 = hidden_states[:split_size], hidden_states[split_size:]
+    residual_1, residual_2 = residual[:split_size], residual[split_size:]
+    blpr_1 = split_size // world_size
+    blpr_2 = hidden_states_2.shape[0] // world_size
+    rows_1 = _shard_rows(split_size, rank, world_size, all_ranks)
+    rows_2 = _shard_rows(hidden_states_2.shape[0], rank, world_size, all_ranks)
+
+    def norm(layernorm, split, max_ctas):
+        hs, res, blpr, off, rows = ((hidden_states_1, residual_1, blpr_1, 0, rows_1) if split == 0 else
+                                    (hidden_states_2, residual_2, blpr_2, offset_second, rows_2))
+        fused_allreduce_layernorm(
+            layernorm=layernorm, hidden_states=hs, residual=res, symm_mem_hdl=symm_mem_hdl,
+            num_tokens_per_rank=blpr, rank=rank, world_size=world_size, MAX_CTAS=max_ctas,
+            offset_symm_mem=off, row_range=rows)
+
+    if layer_id == 0:
+        self.input_layernorm(hidden_states_1, out=residual_1)
+        residual_2.zero_()
+        norm(self.input_layernorm, 1, 8)
+    else:
+        with torch.cuda.stream(copy_stream):
+            copy_stream.wait_stream(current_stream)
+            norm(self.input_layernorm, 1, MAX_CTAS_ATTN)
+
+    with torch.cuda.stream(current_stream):
+        self.self_attn(positions=positions[:split_size], hidden_states=hidden_states_1, split_id=0,
+                       split_size=split_size, num_actual_tokens=split_size)
+        current_stream.wait_stream(copy_stream)
+    with torch.cuda.stream(copy_stream):
+        copy_stream.wait_stream(current_stream)
+        norm(self.post_attention_layernorm, 0, MAX_CTAS_ATTN)
+
+    with torch.cuda.stream(current_stream):
+        self.self_attn(positions=positions[split_size:], hidden_states=hidden_states_2, split_id=1,
+                       split_size=split_size, num_actual_tokens=actual_tokens - split_size)
+        current_stream.wait_stream(copy_stream)
+    with torch.cuda.stream(copy_stream):
+        copy_stream.wait_stream(current_stream)
+        norm(self.post_attention_layernorm, 1, MAX_CTAS_MLP)
+
+    with torch.cuda.stream(current_stream):
+        mlp_fn(hidden_states_1)
+        current_stream.wait_stream(copy_stream)
+    with torch.cuda.stream(copy_stream):
+        copy_stream.wait_stream(current_stream)
+        norm(next_layer_norm, 0, MAX_CTAS_MLP)
+
+    with torch.cuda.stream(current_stream):
+        mlp_fn(hidden_states_2)
+        current_stream.wait_stream(copy_stream)
+
+    if layer_id == end_layer - 1:
+        with torch.cuda.stream(current_stream):
+            norm(next_layer_norm, 1, 16 if actual_tokens < 16384 else 32)
+    return hidden_states, residual

@@ -352,6 +352,15 @@ def main():
                            "gbps": round(c.bytes / r["kernel_us_mean"] / 1e3, 1),
                            "pct_hbm_peak": round(c.bytes / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
             log(f"[sweep] {name}: {sweep[name]}")
+        # Grid-cap sweep of the headline shape (the reference's CTA sweep,
+        # artifact/csvs/figure_10.csv: 2 ... 128 CTAs at 256 rows per GPU).
+        c = cfgs["c2_llama70b_tp8_shard@T256"]
+        cta = {}
+        for cap in (2, 4, 8, 16, 32, 64, 128, 0):
+            r = time_norm(c, 200, 20, cap, device)
+            cta[str(cap or c.T)] = round(r["kernel_us_mean"], 2)
+        sweep["c2_T256_us_by_max_ctas"] = cta
+        log(f"[sweep] c2_T256_us_by_max_ctas: {cta}")
         # The reference's own microbenchmark grid for the P = 1 op (fused_add_rms_norm_cta,
         # H = 8192; artifact/csvs/figure_4.csv, one H100): context, not a baseline for the
         # headline metric, whose P = 8 form the reference does not publish.

@@ -315,7 +315,12 @@ def tokenweave_overlap(
     `input_layernorm(x, out=residual)`; for split 1 the reference reduce-scatters,
     normalises its shard and all-gathers — on one GPU that is the fused op on a
     zeroed residual (residual <- sum of the partials, x <- norm of it).
-    The last layer normalises split 1 after its MLP on the current stream (:327-339)."""
+    The last layer normalises split 1 after its MLP on the current stream (:327-339).
+
+    The two norms that the reference launches with hard-coded grids (8 CTAs in layer
+    0, 16 or 32 after the last layer) have nothing to share the GPU with and are
+    launched uncapped here: on MI355X a compute unit streams at most ~45 GB/s, so a
+    grid of N workgroups is limited to N times that."""
     assert mlp_fn is not None, "mlp_fn must be provided"
     hidden = hidden_states.shape[1]
     offset_second = split_size * hidden * hidden_states.element_size()
@@ -339,7 +344,7 @@ def tokenweave_overlap(
     if layer_id == 0:
         self.input_layernorm(hidden_states_1, out=residual_1)
         residual_2.zero_()
-        norm(self.input_layernorm, 1, 8)
+        norm(self.input_layernorm, 1, 0)
     else:
         with torch.cuda.stream(copy_stream):
             copy_stream.wait_stream(current_stream)
@@ -374,5 +379,5 @@ def tokenweave_overlap(
 
     if layer_id == end_layer - 1:
         with torch.cuda.stream(current_stream):
-            norm(next_layer_norm, 1, 16 if actual_tokens < 16384 else 32)
+            norm(next_layer_norm, 1, 0)
     return hidden_states, residual

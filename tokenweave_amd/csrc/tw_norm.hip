@@ -685,7 +685,8 @@ template <int NP, bool HAS_RES, bool COPY, int Q>
 static int launch_vec(const RowNormArgs& a) {
   const int V = (int)(a.H / 8);
   VecShape sh;
-  if (!vec_shape(V, a.T, &sh)) return 1;  // caller falls back to the element-wise kernel
+  // The shape follows the number of rows in flight: under a grid cap that is the grid.
+  if (!vec_shape(V, a.grid < a.T ? a.grid : a.T, &sh)) return 1;  // caller falls back to the element-wise kernel
   dim3 g(a.grid), b(sh.nt);
   if (a.f16) {
     if (NP != 1) return 1;

@@ -59,6 +59,8 @@ def parse_args():
     ap.add_argument("--max-ctas", type=int, default=0, help="grid cap (0 = library default)")
     ap.add_argument("--sweep", action="store_true", help="also time every configuration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--weave-only", action="store_true",
+                    help="time only the GEMM + norm weave of config 5 and print its figures (for profiling)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="after the timed region, run the library's plain copy kernel on "
                          "buffers of known size (reference traffic for rocprofv3 --pmc runs)")
@@ -308,6 +310,11 @@ def main():
     if args.workload not in cfgs:
         sys.exit(f"unknown workload {args.workload}; choose from {sorted(cfgs)}")
     cfg = cfgs[args.workload]
+    if args.weave_only:
+        w = time_weave(device, norm_cap=0, gemm_cap=128, steps=args.steps)
+        print(json.dumps({"c5_weave": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}}),
+              flush=True)
+        return
     log(f"[bench] {torch.cuda.get_device_name(0)}; workload {cfg.name}: P={cfg.P} T={cfg.T} "
         f"H={cfg.H} bytes/call={cfg.bytes}")
 

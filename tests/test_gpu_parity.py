@@ -450,3 +450,36 @@ def test_bound_ops_equal_the_regular_ops_and_follow_the_given_stream():
     assert torch.equal(out, out_ref)
     with pytest.raises(RuntimeError, match="same shape"):
         ops.bind_reduce_add_rms_norm(inp.partials, y[:10], r, inp.weight, cfg.eps)
+
+
+def _random_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n):
+        P = int(rng.choice([1, 2, 3, 4, 6, 8, 11, 16]))
+        H = 8 * int(rng.integers(1, 1400)) if i % 4 else 8 * int(rng.integers(1400, 5200))
+        T = int(rng.integers(1, 40)) if H > 16384 else int(rng.integers(1, 600))
+        cap = int(rng.choice([0, 0, 1, 3, 17, 100, 1000]))
+        eps = float(rng.choice([1e-5, 1e-6, 1e-3]))
+        scale = float(rng.choice([1e-3, 1.0, 30.0]))
+        cases.append((i, P, T, H, cap, eps, scale))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(48, 20240607), ids=lambda c: f"{c[0]}-P{c[1]}-T{c[2]}-H{c[3]}-cap{c[4]}")
+def test_random_shapes_against_checker(oracle, case):
+    """Seeded random (P, T, H, grid cap, eps, magnitude): every vector-kernel shape, the
+    one-partial-at-a-time path (H > 8192 x 2), run-time P, and the element-wise fallback
+    (H > 32768) against the CPU checker at the tight bar."""
+    i, P, T, H, cap, eps, scale = case
+    print(f"[case] random {case}", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(1000 + i)
+    parts = [(torch.randn(T, H, generator=g, device=DEV) * scale * P ** -0.5).to(torch.bfloat16) for _ in range(P)]
+    r = (torch.randn(T, H, generator=g, device=DEV) * scale).to(torch.bfloat16)
+    w = (1 + 0.2 * torch.randn(H, generator=g, device=DEV)).to(torch.bfloat16)
+    r_want = to_bits(r)
+    y_want, _ = oracle.reduce_add_rms_norm([to_bits(p) for p in parts], r_want, to_bits(w), eps)
+    alias = i % P                      # y overwrites one of the partials
+    ops.reduce_add_rms_norm(parts, parts[alias], r, w, eps, MAX_CTAS=cap or None)
+    torch.cuda.synchronize()
+    assert_parity(to_bits(parts[alias]), to_bits(r), y_want, r_want, f"random case {case}")

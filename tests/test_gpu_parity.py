@@ -483,3 +483,47 @@ def test_random_shapes_against_checker(oracle, case):
     ops.reduce_add_rms_norm(parts, parts[alias], r, w, eps, MAX_CTAS=cap or None)
     torch.cuda.synchronize()
     assert_parity(to_bits(parts[alias]), to_bits(r), y_want, r_want, f"random case {case}")
+
+
+def test_special_values_match_the_checker(oracle):
+    """Infinities, NaNs, overflowing squares, bf16 subnormals and signed zeros: the
+    residual must be the checker's bit for bit (NaN payloads aside), y NaN where it is
+    NaN and within a step elsewhere."""
+    H, P = 1024, 4
+    rows = []
+    base = np.zeros((P + 1, H), np.float32)
+    def row(fill):
+        a = base.copy()
+        fill(a)
+        rows.append(a)
+    row(lambda a: a.__setitem__((0, 3), np.inf))                       # +inf in one partial
+    row(lambda a: (a.__setitem__((0, 3), np.inf), a.__setitem__((1, 3), -np.inf)))   # inf - inf
+    row(lambda a: a.__setitem__((2, 7), np.nan))                       # NaN
+    row(lambda a: a.__setitem__((slice(None), slice(None)), 1e19))     # squares overflow fp32
+    row(lambda a: a.__setitem__((slice(None), slice(None)), 1e-40))    # bf16 / fp32 subnormals
+    row(lambda a: a.__setitem__((P, slice(None)), -0.0))               # negative zeros in the residual
+    row(lambda a: (a.__setitem__((0, slice(None)), 3.0e38), a.__setitem__((1, slice(None)), 3.0e38)))  # sum overflows
+    rng = np.random.default_rng(0)
+    row(lambda a: a.__setitem__((slice(None), slice(None)), rng.standard_normal((P + 1, H)).astype(np.float32)))
+    data = np.stack(rows, axis=1)                                      # [P + 1, T, H]
+    T = data.shape[1]
+    parts = [torch.from_numpy(data[p]).to(DEV).to(torch.bfloat16) for p in range(P)]
+    r = torch.from_numpy(data[P]).to(DEV).to(torch.bfloat16)
+    w = torch.full((H,), 1.5, dtype=torch.bfloat16, device=DEV)
+    r_want = to_bits(r)
+    y_want, _ = oracle.reduce_add_rms_norm([to_bits(p) for p in parts], r_want, to_bits(w), 1e-5)
+    y = torch.empty_like(r)
+    ops.reduce_add_rms_norm(parts, y, r, w, 1e-5)
+    torch.cuda.synchronize()
+    from helpers import bits_to_f32
+    for name, got, want in (("residual", to_bits(r), r_want), ("y", to_bits(y), y_want)):
+        gf, wf = bits_to_f32(got), bits_to_f32(want)
+        assert np.array_equal(np.isnan(gf), np.isnan(wf)), f"{name}: NaN pattern differs"
+        ok = ~np.isnan(wf)
+        if name == "residual":
+            assert np.array_equal(got[ok], want[ok]), f"{name}: bits differ"
+        else:
+            assert ulp_distance(got[ok], want[ok]).max() <= 1, f"{name}: off by more than a step"
+    yw = bits_to_f32(y_want)
+    assert np.isnan(yw[0, 3]) and not np.isnan(yw[0, 4]) and np.isnan(yw[2]).all()   # inf * 0; NaN mean
+    assert (bits_to_f32(y_want)[4] != 0).any(), "subnormal row was flushed by the checker?"

@@ -13,9 +13,10 @@
 //
 // Two kernels:
 //  * gemm_bf16_nt_big_kernel<TM, TN> (K % 64 == 0): (64 TM) x (128 TN) x 64 tiles,
-//    8 waves (2 x 4, two per SIMD), each wave (32 TM) x (32 TN): 192/256/320 x 256
+//    8 waves (2 x 4, two per SIMD), each wave (32 TM) x (32 TN): 128/192/256/320 x 256
 //    (TN = 2) chosen per problem so that the tile count wastes the fewest workgroup
-//    rounds (M = 2458: 320-row tiles make exactly 256 tiles), or 256 x 384.
+//    rounds (M = 2458: 320-row tiles make exactly 256 tiles; M = 1024: 128-row tiles
+//    give every compute unit one), or 256 x 384.
 //    Operand slabs go from global memory straight into LDS (buffer_load ... lds:
 //    no staging registers, no LDS store instructions), two LDS stages.
 //    A wave instruction fills 1 KiB = 8 LDS rows of 128 bytes; row r keeps its
@@ -471,8 +472,9 @@ static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64
 
 // Workgroup tile for the problem, (64 TM) x (128 TN).  Cost = rounds x (tile area /
 // relative throughput + a fixed part per round); ties go to the earlier entry.  The
-// 64-wide wave tiles come in three heights so that a tile count can be made to fit the
-// compute units exactly (M = 2458: 320-row tiles make 256 tiles); 256 x 384 (96-wide
+// 64-wide wave tiles come in four heights so that a tile count can be made to fit the
+// compute units exactly (M = 2458: 320-row tiles make 256 tiles; the 128-row tile loads
+// 30 % more operand bytes per flop than the 192-row one and is rated 0.85); 256 x 384 (96-wide
 // wave tiles, 192 accumulators, exactly 160 KiB of LDS) wins where its fewer, larger
 // rounds fit.  96 x 96 wave tiles (192 x 384) were measured no faster per area than
 // 256 x 256 and are not offered.
@@ -481,7 +483,8 @@ struct BigTile { int tm, tn; };
 static BigTile pick_big_tile(int64_t M, int64_t N, int cus) {
   // Relative throughput per tile area, measured: the 256 x 384 tile loads a fifth fewer
   // operand bytes per flop and runs a round in 1.35x the time of a 256 x 256 round.
-  static const struct { int tm, tn; double eff; } kTiles[] = {{3, 2, 1.0}, {4, 2, 1.0}, {5, 2, 1.0}, {4, 3, 1.1}};
+  static const struct { int tm, tn; double eff; } kTiles[] = {
+      {2, 2, 0.85}, {3, 2, 1.0}, {4, 2, 1.0}, {5, 2, 1.0}, {4, 3, 1.1}};
   BigTile best = {4, 2};
   double best_cost = 1e300;
   for (const auto& t : kTiles) {
@@ -522,6 +525,7 @@ int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t
     int rc;
     const BigTile bt = pick_big_tile(M, N, cus);
     if (bt.tn == 3) rc = launch_big<4, 3>(o, pa, pb, M, N, K, ldc, max_cus, hs);
+    else if (bt.tm == 2) rc = launch_big<2, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
     else if (bt.tm == 3) rc = launch_big<3, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
     else if (bt.tm == 5) rc = launch_big<5, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
     else rc = launch_big<4, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);

@@ -47,6 +47,10 @@ def _require(cond: bool, msg: str) -> None:
 
 
 def _check_tensor(name: str, t: torch.Tensor, dtype: torch.dtype, device: torch.device) -> None:
+    # one pass for the common case; the individual checks below only word the error
+    if (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.device == device
+            and t.is_contiguous()):
+        return
     _require(isinstance(t, torch.Tensor), f"{name} must be a torch.Tensor")
     if not t.is_cuda:
         raise RuntimeError(
@@ -80,26 +84,50 @@ def _require_bf16(name: str, t: torch.Tensor) -> None:
         raise NotImplementedError(f'"{name}" not implemented for \'{t.dtype}\'')
 
 
-def _stream_ptr(t: torch.Tensor) -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+# torch's raw accessors (what its own compiled-kernel launchers use) skip the Stream /
+# device object construction of the public calls; fall back to those if they are gone.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
-class _on_device:
+def _stream_ptr(t: torch.Tensor) -> int:
+    """hipStream_t of the current stream of the tensor's device, as an integer."""
+    if _raw_stream is not None:
+        idx = t.device.index
+        return _raw_stream(idx if idx is not None else torch.cuda.current_device())
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _DeviceGuard:
     """Make the tensor's device current for the duration of the launch
-    (OptionalCUDAGuard in the reference, csrc/tokenweave_fused_kernels.cu:239)."""
+    (OptionalCUDAGuard in the reference, csrc/tokenweave_fused_kernels.cu:239).
+    The usual case — it already is — costs one integer comparison."""
+    __slots__ = ("guard",)
 
-    def __init__(self, t: torch.Tensor):
-        self.idx = t.device.index
+    def __init__(self):
         self.guard = None
 
     def __enter__(self):
-        if self.idx is not None and self.idx != torch.cuda.current_device():
-            self.guard = torch.cuda.device(self.idx)
-            self.guard.__enter__()
+        return self
 
     def __exit__(self, *exc):
         if self.guard is not None:
             self.guard.__exit__(*exc)
+            self.guard = None
+
+
+_NO_SWITCH = _DeviceGuard()
+
+
+def _on_device(t: torch.Tensor):
+    idx = t.device.index
+    cur = _raw_device() if _raw_device is not None else torch.cuda.current_device()
+    if idx is None or idx == cur:
+        return _NO_SWITCH
+    g = _DeviceGuard()
+    g.guard = torch.cuda.device(idx)
+    g.guard.__enter__()
+    return g
 
 
 def _cap(max_ctas: Optional[int]) -> int:
@@ -191,9 +219,8 @@ def _prune_regions() -> None:
 def _peer_stride(mcptr: int, world_size: int) -> int:
     if world_size == 1:
         return 16  # unused: there is only partial 0
-    _prune_regions()
-    for base, stride, slots, _ in _REGIONS:
-        if base <= mcptr < base + stride:
+    for base, stride, slots, owner in _REGIONS:
+        if base <= mcptr < base + stride and owner() is not None:
             _require(world_size <= slots,
                      f"world_size {world_size} exceeds the {slots} slots of the partials region")
             return stride
@@ -250,13 +277,18 @@ class BoundOp:
         self._index = device.index if device.index is not None else torch.cuda.current_device()
 
     def __call__(self, stream: Optional[torch.cuda.Stream] = None) -> None:
-        if stream is None:
-            stream = torch.cuda.current_stream(self._device)
-        if torch.cuda.current_device() != self._index:
-            with torch.cuda.device(self._index):
-                rc = self._fn(*self._args, stream.cuda_stream)
+        if stream is not None:
+            sp = stream.cuda_stream
+        elif _raw_stream is not None:
+            sp = _raw_stream(self._index)
         else:
-            rc = self._fn(*self._args, stream.cuda_stream)
+            sp = torch.cuda.current_stream(self._device).cuda_stream
+        cur = _raw_device() if _raw_device is not None else torch.cuda.current_device()
+        if cur != self._index:
+            with torch.cuda.device(self._index):
+                rc = self._fn(*self._args, sp)
+        else:
+            rc = self._fn(*self._args, sp)
         if rc:
             _lib.check(rc)
 

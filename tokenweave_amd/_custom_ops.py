@@ -66,8 +66,8 @@ def _check_tensor(name: str, t: torch.Tensor, dtype: torch.dtype, device: torch.
 
 def _check_weight(weight: torch.Tensor, hidden: int, dtype, device) -> None:
     _check_tensor("weight", weight, dtype, device)
-    _require(weight.numel() == hidden,
-             f"weight has {weight.numel()} elements, expected hidden_size {hidden}")
+    if weight.numel() != hidden:
+        raise RuntimeError(f"weight has {weight.numel()} elements, expected hidden_size {hidden}")
 
 
 def _dtype_code(name: str, t: torch.Tensor) -> int:
@@ -238,7 +238,8 @@ def _fused_rs_ln(entry: str, kname: str, input, residual, weight, mcptr, signal_
     T, H = _rows(input)
     _require(residual.shape == input.shape, "input and residual must have the same shape")
     _check_weight(weight, H, torch.bfloat16, input.device)
-    _require(0 <= rank < world_size, f"Invalid rank {rank}, must be in [0, {world_size - 1}]")
+    if not 0 <= rank < world_size:
+        raise RuntimeError(f"Invalid rank {rank}, must be in [0, {world_size - 1}]")
     stride = _peer_stride(int(mcptr), int(world_size))
     with _on_device(input):
         _lib.check(getattr(_lib.lib(), entry)(
@@ -304,8 +305,10 @@ def _prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_C
     T, H = _rows(out)
     _require(residual.shape == out.shape, "out and residual must have the same shape")
     for i, p in enumerate(partials):
-        _check_tensor(f"partials[{i}]", p, torch.bfloat16, dev)
-        _require(p.shape == out.shape, f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(out.shape)}")
+        if not (p.is_cuda and p.dtype == torch.bfloat16 and p.device == dev and p.is_contiguous()):
+            _check_tensor(f"partials[{i}]", p, torch.bfloat16, dev)
+        if p.shape != out.shape:
+            raise RuntimeError(f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(out.shape)}")
     _check_weight(weight, H, torch.bfloat16, dev)
     ptrs = (ctypes.c_void_p * P)(*[p.data_ptr() for p in partials])
     args = (ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H, _cap(MAX_CTAS), epsilon)
@@ -335,7 +338,8 @@ FP8_DTYPE = torch.float8_e4m3fn  # gfx950 implements the OCP formats
 
 
 def _check_fp8_out(out: torch.Tensor, like: torch.Tensor) -> None:
-    _require(out.is_cuda and out.device == like.device, f"result is on {out.device}, expected {like.device}")
+    if not (out.is_cuda and out.device == like.device):
+        raise RuntimeError(f"result is on {out.device}, expected {like.device}")
     if out.dtype != FP8_DTYPE:
         raise NotImplementedError(f'"rms_norm_kernel_fp8_type" not implemented for \'{out.dtype}\'')
     _require(out.is_contiguous() and out.shape == like.shape,
@@ -393,7 +397,8 @@ def reduce_add_rms_norm_static_fp8_quant(partials: Sequence[torch.Tensor], resul
     _check_fp8_out(result, residual)
     T, H = _rows(residual)
     for i, p in enumerate(partials):
-        _check_tensor(f"partials[{i}]", p, torch.bfloat16, dev)
+        if not (p.is_cuda and p.dtype == torch.bfloat16 and p.device == dev and p.is_contiguous()):
+            _check_tensor(f"partials[{i}]", p, torch.bfloat16, dev)
         _require(p.shape == residual.shape,
                  f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(residual.shape)}")
     _check_weight(weight, H, torch.bfloat16, dev)
@@ -422,7 +427,8 @@ def _check_dyn_quant(result, like, scales, scale_ub, T):
              "result must be contiguous and have the input's shape")
     _require(scales.is_cuda and scales.device == like.device and scales.dtype == torch.float32,
              "scales must be a float32 tensor on the input's device")
-    _require(scales.is_contiguous() and scales.numel() == T, f"scales must hold {T} contiguous values")
+    if not (scales.is_contiguous() and scales.numel() == T):
+        raise RuntimeError(f"scales must hold {T} contiguous values")
     if scale_ub is not None:
         _require(result.dtype == FP8_DTYPE, "scale_ub is defined for fp8 output only")
         _check_scale(scale_ub, like.device)
@@ -478,8 +484,10 @@ def reduce_add_rms_norm_dynamic_per_token_quant(partials: Sequence[torch.Tensor]
     dev = first.device
     T, H = _rows(first)
     for i, p in enumerate(partials):
-        _check_tensor(f"partials[{i}]", p, torch.bfloat16, dev)
-        _require(p.shape == first.shape, f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(first.shape)}")
+        if not (p.is_cuda and p.dtype == torch.bfloat16 and p.device == dev and p.is_contiguous()):
+            _check_tensor(f"partials[{i}]", p, torch.bfloat16, dev)
+        if p.shape != first.shape:
+            raise RuntimeError(f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(first.shape)}")
     if residual is not None:
         _check_tensor("residual", residual, torch.bfloat16, dev)
         _require(residual.shape == first.shape, "partials and residual must have the same shape")

@@ -453,12 +453,17 @@ static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64
                       int64_t K, int64_t ldc, int max_cus, hipStream_t hs) {
   constexpr int BM = 64 * TM, BN = 128 * TN;
   constexpr int LDS = big_lds_bytes(TM, TN);
-  static std::atomic<bool> lds_ok{false};
-  if (!lds_ok.load(std::memory_order_acquire)) {
+  // the attribute belongs to the function on one device: set it once per device
+  constexpr int kMaxDevices = 64;
+  static std::atomic<bool> lds_ok[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return set_error(TW_ERR_LAUNCH, "gemm_bf16_nt: no current device");
+  if (!lds_ok[dev].load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_big_kernel<TM, TN>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess)
       return set_error(TW_ERR_LAUNCH, "gemm_bf16_nt: the device refused %d bytes of LDS", LDS);
-    lds_ok.store(true, std::memory_order_release);
+    lds_ok[dev].store(true, std::memory_order_release);
   }
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
   int64_t grid = (int64_t)tiles_m * tiles_n;

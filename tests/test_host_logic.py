@@ -223,3 +223,13 @@ def test_fuse_only_schedule_calls_in_reference_order():
     ]
     with pytest.raises(AssertionError, match="mlp_fn"):
         tw.tokenweave_with_fuse_only(Layer(), None, hs, res, object(), 1, nearest_multiple_of_world_size=16)
+
+
+def test_weave_plan_honours_measured_no_overlap_entries():
+    table = {1024: {"attention_ctas": 0, "mlp_ctas": 0, "split_offset": 256, "gemm_cus": 128, "overlap": 0},
+             8192: {"attention_ctas": 0, "mlp_ctas": 0, "split_offset": 256, "gemm_cus": 128, "overlap": 1}}
+    assert tw.weave_plan(1500, table) is None
+    assert tw.weave_plan(8000, table)["gemm_cus"] == 128
+    shipped = tw.load_config()
+    assert all("overlap" in e for e in shipped.values())
+    assert tw.weave_plan(16384, shipped) is not None

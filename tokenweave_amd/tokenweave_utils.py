@@ -51,10 +51,14 @@ def weave_plan(num_tokens: int, config: Dict[int, Dict[str, int]],
                threshold: int = 1024) -> Optional[Dict[str, int]]:
     """What the model forward decides per batch (llama.py:509-521): below `threshold`
     tokens no weave (fuse only) -> None; otherwise the split point and the budgets of
-    the closest table entry."""
+    the closest table entry.  An entry may carry `"overlap": 0` — measured on the
+    target GPU, the two-stream stage was no faster than running its kernels on one
+    stream at that size — which also means fuse only."""
     if num_tokens < threshold:
         return None
     entry = select_config(config, num_tokens)
+    if not entry.get("overlap", 1):
+        return None
     split = min(tokenweave_split_size(num_tokens, entry.get("split_offset", 0)), num_tokens)
     return {"split_size": split, "rest_size": num_tokens - split,
             "attention_ctas": entry.get("attention_ctas", 0), "mlp_ctas": entry.get("mlp_ctas", 0),

@@ -8,7 +8,8 @@ For every token count N and split offset it times the stage the reference overla
 (tokenweave_utils.py:236-260): the row-parallel GEMM [split, K] x [hidden, K]^T of one
 token split on the current stream while the fused P-partial norm of the other split
 runs on a second stream, over a grid of GEMM compute-unit budgets and norm grid caps,
-and keeps the fastest.  The role of artifact/configs_generator/generator.py in the
+and keeps the fastest; the same two kernels are also timed on one stream, and an entry
+whose best weave is not at least 2 % faster gets "overlap": 0 (no weave at that size).  The role of artifact/configs_generator/generator.py in the
 reference, which picks the minimum-latency row of its benchmark sweep.
 """
 from __future__ import annotations
@@ -55,6 +56,32 @@ def time_stage(L, gemm_args, norm_sets, gemm_cus, norm_ctas, steps=40):
     return e0.elapsed_time(e1) * 1e3 / steps
 
 
+def time_serial(L, gemm_args, norm_sets, steps=40):
+    """The same two kernels one after the other on one stream, both uncapped."""
+    s = torch.cuda.Stream()
+    sp = ctypes.c_void_p(s.cuda_stream)
+    out, a, b, M, N, K = gemm_args
+
+    def stage(i):
+        rc = L.tw_gemm_bf16_nt(out, a, b, M, N, K, N, 0, sp)
+        ptrs, P, y, r, w, T, H, eps = norm_sets[i % len(norm_sets)]
+        rc |= L.tw_reduce_add_rms_norm(ptrs, P, y, r, w, T, H, 0, eps, sp)
+        if rc:
+            raise RuntimeError(_lib.last_error())
+
+    with torch.cuda.stream(s):
+        for i in range(5):
+            stage(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(s)
+        for i in range(steps):
+            stage(i)
+        e1.record(s)
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / steps
+
+
 def tune(hidden, k, world_size, tokens, offsets, device="cuda:0", log=print):
     L = _lib.lib()
     cus = ops.num_compute_units(device)
@@ -83,16 +110,19 @@ def tune(hidden, k, world_size, tokens, offsets, device="cuda:0", log=print):
                              inp.weight.data_ptr(), cfg.T, cfg.H, cfg.eps))
             ops.gemm_bf16_nt(out, g.a, g.b)
             gargs = (out.data_ptr(), g.a.data_ptr(), g.b.data_ptr(), split, hidden, k)
+            serial = time_serial(L, gargs, sets)
             for gc in gemm_grid:
                 for nc in norm_grid:
                     us = time_stage(L, gargs, sets, gc, nc)
                     if best is None or us < best[0]:
-                        best = (us, off, gc, nc)
+                        best = (us, off, gc, nc, serial)
             del keep, sets, g, out
             torch.cuda.empty_cache()
-        us, off, gc, nc = best
-        log(f"tokens={n}: best stage {us:.1f} us with split_offset={off} gemm_cus={gc} norm_ctas={nc}")
-        table[str(n)] = {"attention_ctas": nc, "mlp_ctas": nc, "split_offset": off, "gemm_cus": gc}
+        us, off, gc, nc, serial = best
+        log(f"tokens={n}: best stage {us:.1f} us with split_offset={off} gemm_cus={gc} norm_ctas={nc} "
+            f"(one stream: {serial:.1f} us, speedup {serial / us:.2f})")
+        table[str(n)] = {"attention_ctas": nc, "mlp_ctas": nc, "split_offset": off, "gemm_cus": gc,
+                         "overlap": int(us < 0.98 * serial)}
     return table
 
 

@@ -41,13 +41,46 @@ ROTATION_BYTES = 4 << 30      # distinct operand bytes cycled through before any
 
 # HBM bytes per launch read from the hardware counters (rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, each scaled by the same counter's reading for the library's plain copy
-# kernel of known size); the runs are summarised in
-# profiles/row_norm_bf16_c2_T256_pmc_traffic.md.  Workloads without a counter run: None.
-MEASURED_TRAFFIC_BYTES = {"c2_llama70b_tp8_shard@T256": 46366607}
+# kernel of known size), transcribed from the summary named beside each figure; this run
+# does not measure them.  Workloads without a counter run: None.
+MEASURED_TRAFFIC_BYTES = {
+    "c2_llama70b_tp8_shard@T256": (46366607, "profiles/row_norm_bf16_c2_T256_pmc_traffic.md"),
+}
+# dominant kernel of a workload, as rocprofv3 names it
+KERNEL_NAMES = {"c2_llama70b_tp8_shard@T256": "row_norm_bf16_kernel<8,4,256,true,false,0>"}
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+_BENCH_LIB = None
+
+
+def bench_lib():
+    """tokenweave_amd/libtw_bench.so: measurement-only kernels (plain copy, row streams, empty
+    kernel) and the norm kernels compiled with timeline stamps.  Built by `make -C
+    tokenweave_amd/csrc`; the product never loads it."""
+    global _BENCH_LIB
+    if _BENCH_LIB is None:
+        path = os.path.join(ROOT, "tokenweave_amd", "libtw_bench.so")
+        if not os.path.exists(path):
+            sys.exit(f"{path} is missing: build it with `make -C tokenweave_amd/csrc`")
+        L = ctypes.CDLL(path)
+        vp, i64, ci, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+        L.twb_copy_bytes.argtypes = [vp, vp, i64, vp]
+        L.twb_stream_rows.argtypes = [ctypes.POINTER(vp), vp, i64, i64, ci, vp]
+        L.twb_trace_stream_rows.argtypes = [ctypes.POINTER(vp), vp, i64, i64, vp]
+        L.twb_empty.argtypes = [ci, ci, vp]
+        L.twb_trace_reduce_add_rms_norm.argtypes = [ctypes.POINTER(vp), ci, vp, vp, vp, i64, i64, ci, f32, vp, vp]
+        L.tw_last_error.restype = ctypes.c_char_p
+        _BENCH_LIB = L
+    return _BENCH_LIB
+
+
+def bench_check(rc):
+    if rc:
+        raise RuntimeError(bench_lib().tw_last_error().decode())
 
 
 def parse_args():
@@ -64,6 +97,12 @@ def parse_args():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="after the timed region, run the library's plain copy kernel on "
                          "buffers of known size (reference traffic for rocprofv3 --pmc runs)")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="time the memory-system yardsticks (read-only row streams, the norm's traffic "
+                         "without arithmetic, plain copy, empty kernel) at 256 and 2048 rows and print them")
+    ap.add_argument("--timeline", action="store_true",
+                    help="run the workload through the stamped build of the norm kernel and print the "
+                         "per-workgroup timeline breakdown")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline")
     return ap.parse_args()
 
@@ -125,10 +164,20 @@ def quant_bytes(cfg, epilogue):
     return cfg.bytes - cfg.T * cfg.H + (4 * cfg.T if epilogue.endswith("dynamic") else 4)
 
 
-def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16"):
-    """Returns dict(ms_per_step, gbps, kernel_us_mean): wall-clock per step between the
-    two synchronisation points, and the mean launch duration from the HIP events that
-    bracket the same `steps` back-to-back launches."""
+PREROLL_MS = 40.0   # untimed launches ahead of the warm-up: clocks ramped, queues and TLBs in steady state
+REGIONS = 21        # timed regions of exactly `steps` launches each; the median region is reported
+
+
+LEAD_IN = 40        # untimed launches ahead of an event bracket (the bracket starts in a busy queue)
+
+
+def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16", regions=REGIONS, preroll_ms=PREROLL_MS,
+              lead_in=LEAD_IN):
+    """After an untimed pre-roll and `warmup` warm-up launches, times `regions` regions of
+    exactly `steps` back-to-back launches twice over: by the wall clock between two device
+    synchronisations (ms_per_step, gbps), and by HIP events on the launch stream around
+    `steps` launches that follow `lead_in` untimed ones (event_us_per_launch: mean launch
+    duration, gaps included).  Medians over the regions, plus the spread."""
     import torch
     nsets = max(2, min(256, -(-ROTATION_BYTES // cfg.bytes)))
     free, _ = torch.cuda.mem_get_info()
@@ -136,21 +185,48 @@ def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16"):
     nsets = max(2, min(nsets, int(free * 0.6) // (set_bytes * 3)))  # fp32 staging while generating
     runner = NormRunner(cfg, nsets, max_ctas, device, epilogue)
     stream = torch.cuda.current_stream()
-    for i in range(warmup):
-        runner.step(i, stream)
+    it = 0
+    preroll_steps = max(warmup, int(preroll_ms * 1e3 / max(2.0, cfg.bytes / 6e6)))
+    for _ in range(preroll_steps):
+        runner.step(it, stream)
+        it += 1
     torch.cuda.synchronize()
-    # timed region: exactly `steps` launches between two synchronisation points,
-    # bracketed by HIP events on the launch stream
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record(stream)
-    for i in range(steps):
-        runner.step(i, stream)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    for _ in range(warmup):
+        runner.step(it, stream)
+        it += 1
+    # (a) wall clock: exactly `steps` launches between two synchronisations, from an idle queue
+    walls = []
+    for _ in range(regions):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            runner.step(it, stream)
+            it += 1
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - t0)
+    # (b) launch duration: HIP events around exactly `steps` launches that follow `lead_in`
+    # untimed launches on the same stream, so that the bracket starts in a busy queue (what
+    # a per-kernel trace measures) and not with the idle-to-first-dispatch latency
+    events = []
+    for _ in range(regions):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        for _ in range(lead_in):
+            runner.step(it, stream)
+            it += 1
+        e0.record(stream)
+        for _ in range(steps):
+            runner.step(it, stream)
+            it += 1
+        e1.record(stream)
+        torch.cuda.synchronize()
+        events.append(e0.elapsed_time(e1) * 1e-3)
+    wall, ev = statistics.median(walls), statistics.median(events)
     res = {"ms_per_step": wall * 1e3 / steps, "gbps": cfg.bytes * steps / wall / 1e9,
-           "nsets": nsets, "kernel_us_mean": e0.elapsed_time(e1) * 1e3 / steps}
+           "nsets": nsets, "event_us_per_launch": ev * 1e6 / steps,
+           "event_us_per_launch_min": min(events) * 1e6 / steps,
+           "event_us_per_launch_max": max(events) * 1e6 / steps,
+           "regions": regions, "preroll_steps": preroll_steps, "lead_in_steps": lead_in}
     del runner
     torch.cuda.empty_cache()
     return res
@@ -163,15 +239,210 @@ def calibration_copies(device, n=8):
     """n launches of tw_copy_bytes, each reading and writing CALIBRATION_COPY_BYTES of
     memory that was not touched recently (4 source/destination pairs = 2 GiB)."""
     import torch
-    from tokenweave_amd import _custom_ops as ops
+    L = bench_lib()
     pairs = [(torch.ones(CALIBRATION_COPY_BYTES // 2, dtype=torch.bfloat16, device=device),
               torch.empty(CALIBRATION_COPY_BYTES // 2, dtype=torch.bfloat16, device=device))
              for _ in range(4)]
     torch.cuda.synchronize()
+    sp = torch.cuda.current_stream().cuda_stream
     for i in range(n):
         src, dst = pairs[i % 4]
-        ops.copy_bytes(dst, src)
+        bench_check(L.twb_copy_bytes(dst.data_ptr(), src.data_ptr(), CALIBRATION_COPY_BYTES, sp))
     torch.cuda.synchronize()
+
+
+def event_time(fn, steps, stream, warm=20, regions=5):
+    """Median over `regions` of the HIP-event bracket around `steps` back-to-back calls of
+    fn(i), in microseconds per call."""
+    import torch
+    it = 0
+    for _ in range(warm):
+        fn(it)
+        it += 1
+    out = []
+    for _ in range(regions):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(steps):
+            fn(it)
+            it += 1
+        e1.record(stream)
+        torch.cuda.synchronize()
+        out.append(e0.elapsed_time(e1) * 1e3 / steps)
+    return statistics.median(out)
+
+
+def time_ceilings(device):
+    """What the memory system gives kernels with the norm kernel's launch shape (one
+    256-lane workgroup per 16 KiB row, nine input streams, 4 GiB of rotating operands so
+    every launch reads cold HBM), at 256 and 2048 rows of hidden size 8192."""
+    import torch
+    from tokenweave_amd import _lib
+    from tokenweave_amd import workloads as wl
+    L, TL = bench_lib(), _lib.lib()
+    stream = torch.cuda.current_stream()
+    sp = stream.cuda_stream
+    vp = ctypes.c_void_p
+    sink = torch.zeros(4096, dtype=torch.uint8, device=device)
+    out = {}
+    for rows in (256, 2048):
+        cfg = wl.C2.with_tokens(rows)
+        nsets = max(2, min(256, -(-ROTATION_BYTES // cfg.bytes)))
+        sets = []
+        for i in range(nsets):
+            inp = wl.make_norm_inputs(cfg, device, seed_offset=i)
+            ptrs = (vp * 9)(*([p.data_ptr() for p in inp.partials] + [inp.residual.data_ptr()]))
+            sets.append((inp, ptrs))
+        steps = max(50, min(2000, int(0.02 * 5e12 / cfg.bytes)))
+        read_bytes = 9 * rows * cfg.H * 2
+        traffic_bytes = read_bytes + 2 * rows * cfg.H * 2
+        res = {}
+
+        def streams(write):
+            def fn(i):
+                inp, ptrs = sets[i % nsets]
+                bench_check(L.twb_stream_rows(ptrs, sink.data_ptr(), rows, cfg.H, write, sp))
+            return event_time(fn, steps, stream)
+
+        us = streams(0)
+        res["read_only_9_streams"] = {"bytes": read_bytes, "us": round(us, 3), "gbps": round(read_bytes / us / 1e3, 1)}
+        us = streams(1)
+        res["norm_traffic_no_arithmetic"] = {"bytes": traffic_bytes, "us": round(us, 3),
+                                             "gbps": round(traffic_bytes / us / 1e3, 1)}
+        us = streams(2)
+        res["write_only_2_streams"] = {"bytes": traffic_bytes - read_bytes, "us": round(us, 3),
+                                       "gbps": round((traffic_bytes - read_bytes) / us / 1e3, 1)}
+        # plain copy moving the same number of bytes in total (half read, half written)
+        half = (traffic_bytes // 2) // 16 * 16
+        srcs = [inp.staging.view(-1).view(torch.uint8) for inp, _ in sets]
+        dsts = [torch.empty(half, dtype=torch.uint8, device=device) for _ in range(min(nsets, 8))]
+
+        def copy(i):
+            bench_check(L.twb_copy_bytes(dsts[i % len(dsts)].data_ptr(), srcs[i % nsets].data_ptr(), half, sp))
+        us = event_time(copy, steps, stream)
+        res["plain_copy_same_total_bytes"] = {"bytes": 2 * half, "us": round(us, 3),
+                                              "gbps": round(2 * half / us / 1e3, 1)}
+
+        def norm(i):
+            inp, ptrs = sets[i % nsets]
+            rc = TL.tw_reduce_add_rms_norm(ctypes.cast(ptrs, ctypes.POINTER(vp)), cfg.P, inp.partials[0].data_ptr(),
+                                           inp.residual.data_ptr(), inp.weight.data_ptr(), cfg.T, cfg.H, 0,
+                                           cfg.eps, sp)
+            if rc:
+                _lib.check(rc)
+        us = event_time(norm, steps, stream)
+        res["norm_kernel"] = {"bytes": cfg.bytes, "us": round(us, 3), "gbps": round(cfg.bytes / us / 1e3, 1)}
+        us = event_time(lambda i: bench_check(L.twb_empty(rows, 256, sp)), 2000, stream)
+        res["empty_kernel_same_grid"] = {"us": round(us, 3)}
+        out[f"rows{rows}"] = res
+        log(f"[ceilings] rows={rows}: {res}")
+        del sets, srcs, dsts
+        torch.cuda.empty_cache()
+    return out
+
+
+def time_timeline(cfg, device, launches=200):
+    """Runs the stamped build of the norm kernel `launches` times on rotating inputs and
+    reduces the per-row stamps (wall clock, 10 ns units) to a breakdown of one launch:
+    microseconds; `min`/`median`/`max` are over the rows of a launch, each then the
+    median over launches."""
+    import numpy as np
+    import torch
+    from tokenweave_amd import workloads as wl
+    L = bench_lib()
+    stream = torch.cuda.current_stream()
+    sp = stream.cuda_stream
+    vp = ctypes.c_void_p
+    nsets = max(2, min(256, -(-ROTATION_BYTES // cfg.bytes)))
+    sets = []
+    for i in range(nsets):
+        inp = wl.make_norm_inputs(cfg, device, seed_offset=i)
+        sets.append((inp, (vp * cfg.P)(*[p.data_ptr() for p in inp.partials])))
+    trace = torch.zeros((launches, cfg.T, 8), dtype=torch.int64, device=device)
+
+    def call(i, slot):
+        inp, ptrs = sets[i % nsets]
+        bench_check(L.twb_trace_reduce_add_rms_norm(ptrs, cfg.P, inp.partials[0].data_ptr(),
+                                                    inp.residual.data_ptr(), inp.weight.data_ptr(), cfg.T, cfg.H,
+                                                    0, cfg.eps, trace[slot].data_ptr(), sp))
+    for i in range(50):
+        call(i, 0)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for i in range(launches):
+        call(50 + i, i)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    event_us = e0.elapsed_time(e1) * 1e3 / launches
+    t = trace.cpu().numpy()
+    st = t[:, :, :6].astype(np.float64) * 0.01          # 100 MHz wall clock -> us
+    xcc = (t[:, :, 6] >> 32) & 0xf
+    rel = st - st[:, :, 0].min(axis=1)[:, None, None]   # relative to the launch's first row begin
+
+    def med(a):
+        return float(np.median(a))
+
+    def rows_stat(a):
+        return {"min": round(med(a.min(axis=1)), 2), "median": round(med(np.median(a, axis=1)), 2),
+                "max": round(med(a.max(axis=1)), 2)}
+    span = rel[:, :, 5].max(axis=1)
+    gaps = st[1:, :, 0].min(axis=1) - st[:-1, :, 5].max(axis=1)
+    out = {
+        "workload": cfg.name, "launches": launches,
+        "event_us_per_launch_with_stamps": round(event_us, 3),
+        "first_row_begin_to_last_ack_us": {"median": round(med(span), 2), "min": round(float(span.min()), 2),
+                                           "max": round(float(span.max()), 2)},
+        "last_ack_to_next_launch_first_row_us": {"median": round(med(gaps), 2), "min": round(float(gaps.min()), 2),
+                                                 "max": round(float(gaps.max()), 2)},
+        "row_begin_after_first_row_us": rows_stat(rel[:, :, 0]),
+        "loads_returned_after_row_begin_us": rows_stat(st[:, :, 1] - st[:, :, 0]),
+        "loads_returned_after_first_row_us": rows_stat(rel[:, :, 1]),
+        "residual_stores_issued_after_loads_us": rows_stat(st[:, :, 2] - st[:, :, 1]),
+        "row_sum_after_residual_stores_us": rows_stat(st[:, :, 3] - st[:, :, 2]),
+        "y_stores_issued_after_row_sum_us": rows_stat(st[:, :, 4] - st[:, :, 3]),
+        "stores_acknowledged_after_y_issue_us": rows_stat(st[:, :, 5] - st[:, :, 4]),
+        "row_end_after_first_row_us": rows_stat(rel[:, :, 5]),
+        "rows_per_xcc_first_launch": [int((xcc[0] == x).sum()) for x in range(8)],
+        "median_row_end_by_xcc_us": [round(med(rel[:, :, 5][xcc == x]), 2) if (xcc == x).any() else None
+                                     for x in range(8)],
+    }
+    return out
+
+
+def time_arrivals(cfg, device, launches=100):
+    """The stand-in kernel (the norm's traffic, no arithmetic) with a stamp after each of
+    the nine streams has returned: when, after the launch's first row begins, the data
+    of a row arrives.  Microseconds; min / median / max over the rows of a launch, each
+    the median over launches."""
+    import numpy as np
+    import torch
+    from tokenweave_amd import workloads as wl
+    L = bench_lib()
+    stream = torch.cuda.current_stream()
+    sp = stream.cuda_stream
+    vp = ctypes.c_void_p
+    nsets = max(2, min(256, -(-ROTATION_BYTES // cfg.bytes)))
+    sets = []
+    for i in range(nsets):
+        inp = wl.make_norm_inputs(cfg, device, seed_offset=i)
+        sets.append((inp, (vp * 9)(*([p.data_ptr() for p in inp.partials] + [inp.residual.data_ptr()]))))
+    trace = torch.zeros((launches, cfg.T, 16), dtype=torch.int64, device=device)
+    for i in range(launches + 20):
+        inp, ptrs = sets[i % nsets]
+        bench_check(L.twb_trace_stream_rows(ptrs, trace[max(0, i - 20)].data_ptr(), cfg.T, cfg.H, sp))
+    torch.cuda.synchronize()
+    st = trace.cpu().numpy()[:, :, :12].astype(np.float64) * 0.01
+    rel = st - st[:, :, 0].min(axis=1)[:, None, None]
+    names = ["row_begins"] + [f"stream_{s}_returned" for s in range(9)] + ["stores_issued", "stores_acknowledged"]
+    out = {"workload": cfg.name, "launches": launches}
+    for j, n in enumerate(names):
+        a = rel[:, :, j]
+        out[n] = {"min": round(float(np.median(a.min(axis=1))), 2),
+                  "median": round(float(np.median(np.median(a, axis=1))), 2),
+                  "max": round(float(np.median(a.max(axis=1))), 2)}
+    return out
 
 
 def time_norm_warm(cfg, steps, max_ctas, device):
@@ -310,6 +581,13 @@ def main():
     if args.workload not in cfgs:
         sys.exit(f"unknown workload {args.workload}; choose from {sorted(cfgs)}")
     cfg = cfgs[args.workload]
+    if args.ceilings:
+        print(json.dumps({"ceilings": time_ceilings(device)}), flush=True)
+        return
+    if args.timeline:
+        print(json.dumps({"timeline": time_timeline(cfg, device), "arrivals": time_arrivals(cfg, device)}),
+              flush=True)
+        return
     if args.weave_only:
         w = time_weave(device, norm_cap=0, gemm_cap=128, steps=args.steps)
         print(json.dumps({"c5_weave": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}}),
@@ -320,7 +598,8 @@ def main():
 
     res = time_norm(cfg, args.steps, args.warmup, args.max_ctas, device)
     log(f"[bench] {res}")
-    kernel_us = res["kernel_us_mean"]
+    kernel_us = res["event_us_per_launch"]
+    traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name, (None, None)) if args.max_ctas == 0 else (None, None)
     achieved = cfg.bytes / kernel_us / 1e3
     out = {
         "metric": "fused P-partial reduce+add+RMSNorm GB/s (% HBM peak), us/call, H=8192",
@@ -330,14 +609,21 @@ def main():
         "data": "synthetic",
         "config": {"workload": cfg.name, "P": cfg.P, "T": cfg.T, "H": cfg.H, "eps": cfg.eps,
                    "bytes_per_call": cfg.bytes, "rotating_input_sets": res["nsets"],
-                   "max_ctas": args.max_ctas},
+                   "max_ctas": args.max_ctas, "timed_regions": res["regions"],
+                   "region_reported": "median", "preroll_steps": res["preroll_steps"]},
         "pct_hbm_peak": round(100.0 * res["gbps"] / HBM_PEAK_GBPS, 2),
         "us_per_call": round(res["ms_per_step"] * 1e3, 3),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name) if args.max_ctas == 0 else None,
-                     "kernel": "row_norm_bf16_kernel<8,4,256,true,false,0>",
-                     "kernel_us_mean": round(kernel_us, 3)},
+                     "traffic": traffic[0], "traffic_source": traffic[1],
+                     "kernel": KERNEL_NAMES.get(cfg.name),
+                     "duration_source": "HIP-event bracket around each region's `steps` launches on the "
+                                        "launch stream, after `lead_in_steps` untimed launches (launch gaps "
+                                        "included), median region",
+                     "lead_in_steps": res["lead_in_steps"],
+                     "event_us_per_launch": round(kernel_us, 3),
+                     "event_us_per_launch_min_max": [round(res["event_us_per_launch_min"], 3),
+                                                     round(res["event_us_per_launch_max"], 3)]},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
@@ -350,22 +636,22 @@ def main():
         cfgs["c2_unsharded@T2048"] = wl.C2.with_tokens(2048, "c2_unsharded@T2048")
         for name, c in cfgs.items():
             steps = max(50, min(2000, int(0.02 * 5e12 / c.bytes)))  # ~20 ms of kernel time
-            r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device)
+            r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device, regions=5, preroll_ms=10.0)
             warm_us = time_norm_warm(c, steps, args.max_ctas, device) if c.bytes < (200 << 20) else None
             sweep[name] = {"P": c.P, "T": c.T, "H": c.H, "bytes": c.bytes,
                            "us_per_call": round(r["ms_per_step"] * 1e3, 3),
-                           "kernel_us": round(r["kernel_us_mean"], 3),
+                           "kernel_us": round(r["event_us_per_launch"], 3),
                            "kernel_us_cache_resident": None if warm_us is None else round(warm_us, 3),
-                           "gbps": round(c.bytes / r["kernel_us_mean"] / 1e3, 1),
-                           "pct_hbm_peak": round(c.bytes / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
+                           "gbps": round(c.bytes / r["event_us_per_launch"] / 1e3, 1),
+                           "pct_hbm_peak": round(c.bytes / r["event_us_per_launch"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
             log(f"[sweep] {name}: {sweep[name]}")
         # Grid-cap sweep of the headline shape (the reference's CTA sweep,
         # artifact/csvs/figure_10.csv: 2 ... 128 CTAs at 256 rows per GPU).
         c = cfgs["c2_llama70b_tp8_shard@T256"]
         cta = {}
         for cap in (2, 4, 8, 16, 32, 64, 128, 0):
-            r = time_norm(c, 200, 20, cap, device)
-            cta[str(cap or c.T)] = round(r["kernel_us_mean"], 2)
+            r = time_norm(c, 200, 20, cap, device, regions=5, preroll_ms=10.0)
+            cta[str(cap or c.T)] = round(r["event_us_per_launch"], 2)
         sweep["c2_T256_us_by_max_ctas"] = cta
         log(f"[sweep] c2_T256_us_by_max_ctas: {cta}")
         # The reference's own microbenchmark grid for the P = 1 op (fused_add_rms_norm_cta,
@@ -375,22 +661,22 @@ def main():
                               (32768, 712.4)):
             c = wl.C1.with_tokens(rows, f"p1_add_rms_norm@T{rows}")
             steps = max(50, min(2000, int(0.02 * 5e12 / c.bytes)))
-            r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device)
+            r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device, regions=5, preroll_ms=10.0)
             sweep[c.name] = {"P": 1, "T": rows, "H": c.H, "bytes": c.bytes,
-                             "kernel_us": round(r["kernel_us_mean"], 3),
-                             "gbps": round(c.bytes / r["kernel_us_mean"] / 1e3, 1),
-                             "pct_hbm_peak": round(c.bytes / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2),
+                             "kernel_us": round(r["event_us_per_launch"], 3),
+                             "gbps": round(c.bytes / r["event_us_per_launch"] / 1e3, 1),
+                             "pct_hbm_peak": round(c.bytes / r["event_us_per_launch"] / 1e3 / HBM_PEAK_GBPS * 100, 2),
                              "reference_h100_us": h100_us}
             log(f"[sweep] {c.name}: {sweep[c.name]}")
         for name in ("c2_llama70b_tp8_shard@T256", "c2_unsharded@T2048"):
             c = cfgs[name]
             steps = max(50, min(2000, int(0.02 * 5e12 / c.bytes)))
             for epi in ("fp8_static", "fp8_dynamic", "int8_dynamic"):
-                r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device, epi)
+                r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device, epi, regions=5, preroll_ms=10.0)
                 b = quant_bytes(c, epi)
-                sweep[f"{name}+{epi}"] = {"bytes": b, "kernel_us": round(r["kernel_us_mean"], 3),
-                                          "gbps": round(b / r["kernel_us_mean"] / 1e3, 1),
-                                          "pct_hbm_peak": round(b / r["kernel_us_mean"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
+                sweep[f"{name}+{epi}"] = {"bytes": b, "kernel_us": round(r["event_us_per_launch"], 3),
+                                          "gbps": round(b / r["event_us_per_launch"] / 1e3, 1),
+                                          "pct_hbm_peak": round(b / r["event_us_per_launch"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
                 log(f"[sweep] {name}+{epi}: {sweep[f'{name}+{epi}']}")
         w = time_weave(device, norm_cap=0, gemm_cap=128)
         sweep["c5_weave"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}

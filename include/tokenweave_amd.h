@@ -134,6 +134,47 @@ TW_API int tw_fused_rs_ln_ag_cta(void* input, void* residual, const void* weight
                           int64_t num_tokens, int64_t hidden_size,
                           void* stream);
 
+/* Workspace of the *_ws entry points: TW_SPLIT_WORKSPACE_BYTES of device memory,
+ * 256-byte aligned, all zeros before the first call that uses it.  Every call
+ * leaves it ready for the next one (its arrival counters back at zero) when its
+ * kernel has finished.  Calls that share a workspace must not overlap in time
+ * (same stream, or ordered by events). */
+#define TW_SPLIT_MAX_TOKENS 256
+#define TW_SPLIT_WORKSPACE_BYTES (TW_SPLIT_MAX_TOKENS * 384)
+
+/* tw_reduce_add_rms_norm for decode-size batches.  With few token rows and many
+ * compute units a row is cut into segments of whole 64-vector chunks, one
+ * workgroup per segment; the segments leave their partial sums of squares in
+ * `workspace`, and the workgroup that arrives last normalises the row.  Results
+ * are bit-identical to tw_reduce_add_rms_norm.  The split is used when
+ * max_ctas <= 0, num_tokens <= TW_SPLIT_MAX_TOKENS and tw_split_segments() says
+ * more than one segment; otherwise, or with workspace == NULL, the call IS
+ * tw_reduce_add_rms_norm.  workspace_bytes < TW_SPLIT_WORKSPACE_BYTES is an error.
+ * The reference sizes its persistent grids per batch so that its kernels are not
+ * starved of CTAs (grid = min(MAX_CTAS, rows), block = hidden_size / 8:
+ * csrc/tokenweave_fused_kernels.cu:241-244, vllm/model_executor/models/
+ * tokenweave_utils.py:86); on 256 compute units a decode batch of 1-32 rows needs
+ * more than one workgroup per row to do the same. */
+TW_API int tw_reduce_add_rms_norm_ws(const void* const* partials, int num_partials,
+                              void* y, void* residual, const void* weight,
+                              int64_t num_tokens, int64_t hidden_size,
+                              int max_ctas, float epsilon, void* workspace,
+                              int64_t workspace_bytes, void* stream);
+
+/* tw_fused_rs_ln_ag_cta (= tw_fused_rs_ln_cta on one GPU) with the workspace of
+ * tw_reduce_add_rms_norm_ws: the reference's argument list for decode-size
+ * batches.  Replaces ::fused_rs_ln_ag_cta / ::fused_rs_ln_cta as above. */
+TW_API int tw_fused_rs_ln_ag_cta_ws(void* input, void* residual, const void* weight,
+                             uint64_t mcptr, int64_t peer_stride_bytes, int rank,
+                             int world_size, int max_ctas, float epsilon,
+                             int64_t num_tokens, int64_t hidden_size,
+                             void* workspace, int64_t workspace_bytes,
+                             void* stream);
+
+/* Segments per row the *_ws entry points use for this shape on the current
+ * device: 1 = one workgroup per row (no workspace traffic). */
+TW_API int tw_split_segments(int64_t num_tokens, int64_t hidden_size, int max_ctas);
+
 /* out[M, N] = a[M, K] * b[N, K]^T, bf16 in, fp32 accumulate on MFMA, bf16 out.
  * `ldc` is the row stride of out in elements (>= N), so the result can land in
  * a row slice of a wider staging buffer.  Required: K % 8 == 0, N % 4 == 0,
@@ -205,13 +246,6 @@ TW_API int tw_reduce_add_rms_norm_dynamic_per_token_quant(
     const void* const* partials, int num_partials, void* out, float* scales, void* residual,
     const void* weight, const float* scale_ub, int64_t num_tokens, int64_t hidden_size,
     int max_ctas, float epsilon, int out_kind, void* stream);
-
-/* dst[0, nbytes) <- src[0, nbytes) with a plain grid-stride copy kernel (default
- * cache policy, 16 bytes per lane).  nbytes % 16 == 0, 16-byte aligned pointers,
- * non-overlapping ranges.  A measurement utility with no counterpart in the
- * reference: its traffic is known exactly, so hardware memory counters read for
- * the norm kernels can be scaled against it. */
-TW_API int tw_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream);
 
 #ifdef __cplusplus
 }

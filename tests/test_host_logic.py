@@ -121,17 +121,27 @@ def test_rmsnorm_module_surface_and_native_path():
 def test_partials_region_lookup():
     class Owner:
         pass
-    o = Owner()
-    ops.register_partials_region(0x10000, 0x1000, 8, o)
-    assert ops._peer_stride(0x10000 + 0x800, 8) == 0x1000
+    o, o2 = Owner(), Owner()
+    ops.register_partials_region(0x10000, 0x1000, 8, o, usable_bytes=0xC00)
+    ops.register_partials_region(0x40000, 0x2000, 4, o2)
+    assert ops._peer_stride(0x10000 + 0x800, 8, 0x400) == 0x1000
+    assert ops._peer_stride(0x40000, 4, 0x2000) == 0x2000          # the other region, then back
+    assert ops._peer_stride(0x10000, 8, 0xC00) == 0x1000
     with pytest.raises(RuntimeError, match="not inside slot 0"):
-        ops._peer_stride(0x10000 + 0x1000, 8)
+        ops._peer_stride(0x10000 + 0x1000, 8, 16)
     with pytest.raises(RuntimeError, match="exceeds the 8 slots"):
-        ops._peer_stride(0x10000, 9)
-    assert ops._peer_stride(0xdead0, 1) == 16
+        ops._peer_stride(0x10000, 9, 16)
+    # the rows a call reads must stay inside the usable part of a slot (a too large
+    # hidden_states or offset would read past the staging buffer of the last rank)
+    with pytest.raises(RuntimeError, match="reach past the 3072 usable bytes"):
+        ops._peer_stride(0x10000 + 0x800, 8, 0x401)
+    with pytest.raises(RuntimeError, match="reach past"):
+        ops._peer_stride(0x40000 + 0x1000, 4, 0x1010)
+    assert ops._peer_stride(0xdead0, 1, 1 << 40) == 16
     del o
     with pytest.raises(RuntimeError, match="not inside slot 0"):
-        ops._peer_stride(0x10000, 8)
+        ops._peer_stride(0x10000, 8, 16)
+    assert ops._peer_stride(0x40000, 4, 16) == 0x2000
 
 
 def test_algorithmic_bytes_table():

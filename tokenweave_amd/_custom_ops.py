@@ -13,9 +13,11 @@ an op with CPU tensors, or without the built library, raises.
 """
 from __future__ import annotations
 
+import bisect
 import ctypes
+import threading
 import weakref
-from typing import List, Optional, Sequence, Tuple
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -200,33 +202,88 @@ def fused_add_rms_norm_cta(input: torch.Tensor, residual: torch.Tensor, weight: 
 # in every rank's staging buffer (layernorm.py:79).  On one GPU the P staging
 # buffers are slots of one allocation; a registered region tells the shim the
 # distance between slots so that `mcptr + p * stride` is partial p.
-_REGIONS: List[Tuple[int, int, int, "weakref.ref"]] = []  # (base, stride_bytes, slots, owner)
+# Regions are kept sorted by base address (bisect) behind a lock; the region that served
+# the last call is tried first, so the usual lookup is a few comparisons.
+_REGIONS: List[Tuple[int, int, int, int, "weakref.ref"]] = []  # (base, stride, slots, usable, owner)
+_REGION_BASES: List[int] = []
+_REGIONS_LOCK = threading.Lock()
+_LAST_REGION: Optional[Tuple[int, int, int, int, "weakref.ref"]] = None
 
 
-def register_partials_region(base_ptr: int, stride_bytes: int, slots: int, owner) -> None:
+def register_partials_region(base_ptr: int, stride_bytes: int, slots: int, owner,
+                             usable_bytes: Optional[int] = None) -> None:
     """Declare [base_ptr, base_ptr + slots*stride_bytes) as `slots` equally spaced
-    partial-sum buffers.  `owner` is weakly referenced; the region is dropped with it."""
+    partial-sum buffers of `usable_bytes` each (default: the whole stride).  `owner` is
+    weakly referenced; the region is dropped with it."""
+    global _LAST_REGION
     _require(stride_bytes > 0 and stride_bytes % 16 == 0, "slot stride must be a positive multiple of 16")
     _require(1 <= slots <= _lib.TW_MAX_PARTIALS, f"slots must be in [1, {_lib.TW_MAX_PARTIALS}]")
-    _prune_regions()
-    _REGIONS.append((int(base_ptr), int(stride_bytes), int(slots), weakref.ref(owner)))
+    usable = int(stride_bytes if usable_bytes is None else usable_bytes)
+    _require(0 < usable <= stride_bytes, "usable bytes of a slot must fit its stride")
+    entry = (int(base_ptr), int(stride_bytes), int(slots), usable, weakref.ref(owner))
+    with _REGIONS_LOCK:
+        live = [r for r in _REGIONS if r[4]() is not None and r[0] != entry[0]]
+        live.append(entry)
+        live.sort(key=lambda r: r[0])
+        _REGIONS[:] = live
+        _REGION_BASES[:] = [r[0] for r in live]
+        _LAST_REGION = None
 
 
-def _prune_regions() -> None:
-    _REGIONS[:] = [r for r in _REGIONS if r[3]() is not None]
+def _find_region(mcptr: int):
+    global _LAST_REGION
+    r = _LAST_REGION
+    if r is not None and r[0] <= mcptr < r[0] + r[1] and r[4]() is not None:
+        return r
+    with _REGIONS_LOCK:
+        i = bisect.bisect_right(_REGION_BASES, mcptr) - 1
+        if i >= 0:
+            r = _REGIONS[i]
+            if r[0] <= mcptr < r[0] + r[1] and r[4]() is not None:
+                _LAST_REGION = r
+                return r
+    return None
 
 
-def _peer_stride(mcptr: int, world_size: int) -> int:
+def _peer_stride(mcptr: int, world_size: int, nbytes: int) -> int:
+    """Distance between the partial buffers that `mcptr` addresses, after checking that
+    the `nbytes` the kernel reads from every slot lie inside the slot."""
     if world_size == 1:
         return 16  # unused: there is only partial 0
-    for base, stride, slots, owner in _REGIONS:
-        if base <= mcptr < base + stride and owner() is not None:
-            _require(world_size <= slots,
-                     f"world_size {world_size} exceeds the {slots} slots of the partials region")
-            return stride
-    raise RuntimeError(
-        f"mcptr 0x{mcptr:x} is not inside slot 0 of a registered partials region "
-        "(allocate the staging buffers with tokenweave_amd.PartialsBuffer)")
+    r = _find_region(mcptr)
+    if r is None:
+        raise RuntimeError(
+            f"mcptr 0x{mcptr:x} is not inside slot 0 of a registered partials region "
+            "(allocate the staging buffers with tokenweave_amd.PartialsBuffer)")
+    base, stride, slots, usable, _ = r
+    _require(world_size <= slots,
+             f"world_size {world_size} exceeds the {slots} slots of the partials region")
+    if (mcptr - base) + nbytes > usable:
+        raise RuntimeError(
+            f"the rows of this call ({nbytes} bytes at offset {mcptr - base}) reach past the "
+            f"{usable} usable bytes of a staging slot")
+    return stride
+
+
+# --- workspace of the split-row kernel (decode-size batches) -------------------
+# One zeroed TW_SPLIT_WORKSPACE_BYTES buffer per (device, stream): calls on one stream
+# are ordered, which is what sharing a workspace requires.  Allocated on the first
+# small-batch call on that stream and kept for the life of the process.
+_SPLIT_WS: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def split_workspace(device_index: int, stream_ptr: int) -> torch.Tensor:
+    ws = _SPLIT_WS.get((device_index, stream_ptr))
+    if ws is None:
+        ws = torch.zeros(_lib.TW_SPLIT_WORKSPACE_BYTES, dtype=torch.uint8,
+                         device=torch.device("cuda", device_index))
+        assert ws.data_ptr() % 256 == 0
+        _SPLIT_WS[(device_index, stream_ptr)] = ws
+    return ws
+
+
+def _wants_split(T: int, cap: int) -> bool:
+    return cap <= 0 and 0 < T <= _lib.TW_SPLIT_MAX_TOKENS
 
 
 def _fused_rs_ln(entry: str, kname: str, input, residual, weight, mcptr, signal_pads, rank,
@@ -240,11 +297,20 @@ def _fused_rs_ln(entry: str, kname: str, input, residual, weight, mcptr, signal_
     _check_weight(weight, H, torch.bfloat16, input.device)
     if not 0 <= rank < world_size:
         raise RuntimeError(f"Invalid rank {rank}, must be in [0, {world_size - 1}]")
-    stride = _peer_stride(int(mcptr), int(world_size))
+    stride = _peer_stride(int(mcptr), int(world_size), T * H * 2)
+    cap = _cap(MAX_CTAS)
     with _on_device(input):
+        sp = _stream_ptr(input)
+        if _wants_split(T, cap):
+            idx = input.device.index
+            ws = split_workspace(torch.cuda.current_device() if idx is None else idx, sp)
+            _lib.check(_lib.lib().tw_fused_rs_ln_ag_cta_ws(
+                input.data_ptr(), residual.data_ptr(), weight.data_ptr(), int(mcptr), stride,
+                int(rank), int(world_size), cap, epsilon, T, H, ws.data_ptr(), ws.numel(), sp))
+            return
         _lib.check(getattr(_lib.lib(), entry)(
             input.data_ptr(), residual.data_ptr(), weight.data_ptr(), int(mcptr), stride,
-            int(rank), int(world_size), _cap(MAX_CTAS), epsilon, T, H, _stream_ptr(input)))
+            int(rank), int(world_size), cap, epsilon, T, H, sp))
 
 
 def fused_rs_ln_ag_cta(input: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,
@@ -294,7 +360,7 @@ class BoundOp:
             _lib.check(rc)
 
 
-def _prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS):
+def _prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS, split=None):
     P = len(partials)
     _require(1 <= P <= _lib.TW_MAX_PARTIALS,
              f"number of partials {P} not in [1, {_lib.TW_MAX_PARTIALS}]")
@@ -311,23 +377,48 @@ def _prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_C
             raise RuntimeError(f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(out.shape)}")
     _check_weight(weight, H, torch.bfloat16, dev)
     ptrs = (ctypes.c_void_p * P)(*[p.data_ptr() for p in partials])
-    args = (ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H, _cap(MAX_CTAS), epsilon)
+    cap = _cap(MAX_CTAS)
+    if _wants_split(T, cap) if split is None else split:
+        # decode-size batch: the split-row kernel, with a workspace of the op's own (a bound
+        # op may be launched on any stream, but not on two at once)
+        ws = torch.zeros(_lib.TW_SPLIT_WORKSPACE_BYTES, dtype=torch.uint8, device=dev)
+        args = (ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H, cap, epsilon,
+                ws.data_ptr(), ws.numel())
+        return _lib.lib().tw_reduce_add_rms_norm_ws, args, (list(partials), out, residual, weight, ws), dev
+    args = (ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H, cap, epsilon)
     return _lib.lib().tw_reduce_add_rms_norm, args, (list(partials), out, residual, weight), dev
 
 
 def reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
                         residual: torch.Tensor, weight: torch.Tensor, epsilon: float,
-                        MAX_CTAS: Optional[int] = None) -> None:
+                        MAX_CTAS: Optional[int] = None, split: Optional[bool] = None) -> None:
     """out <- RMSNorm(sum_p partials[p] + residual) * weight; residual <- the sum.
-    `out` may be one of the partials."""
-    BoundOp(*_prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS))()
+    `out` may be one of the partials.  Uncapped calls of at most TW_SPLIT_MAX_TOKENS rows
+    go through the split-row entry point (several workgroups per row, same bits);
+    `split=False` forces the one-workgroup-per-row kernel."""
+    fn, args, keep, dev = _prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS,
+                                                       False)
+    if (_wants_split(args[5], args[7]) if split is None else split):
+        idx = dev.index if dev.index is not None else torch.cuda.current_device()
+        with _on_device(out):
+            sp = _stream_ptr(out)
+            ws = split_workspace(idx, sp)
+            _lib.check(_lib.lib().tw_reduce_add_rms_norm_ws(*args, ws.data_ptr(), ws.numel(), sp))
+        return
+    BoundOp(fn, args, keep, dev)()
 
 
 def bind_reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
                              residual: torch.Tensor, weight: torch.Tensor, epsilon: float,
-                             MAX_CTAS: Optional[int] = None) -> BoundOp:
+                             MAX_CTAS: Optional[int] = None, split: Optional[bool] = None) -> BoundOp:
     """`reduce_add_rms_norm` with the checks done now and the launch deferred."""
-    return BoundOp(*_prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS))
+    return BoundOp(*_prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS, split))
+
+
+def split_segments(num_tokens: int, hidden_size: int, MAX_CTAS: Optional[int] = None) -> int:
+    """Workgroups per row the split-row entry points use for this shape on the current
+    device (1 = one workgroup per row)."""
+    return _lib.lib().tw_split_segments(num_tokens, hidden_size, _cap(MAX_CTAS))
 
 
 # ---------------------------------------------------------------------------
@@ -532,16 +623,6 @@ def bind_gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
                       max_cus: Optional[int] = None) -> BoundOp:
     """`gemm_bf16_nt` with the checks done now and the launch deferred."""
     return BoundOp(*_prepare_gemm_bf16_nt(out, a, b, max_cus))
-
-
-def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
-    """dst <- src through the library's plain copy kernel (counter calibration)."""
-    _require(dst.is_cuda and src.is_cuda and dst.device == src.device, "copy needs two tensors on one GPU")
-    _require(dst.is_contiguous() and src.is_contiguous(), "copy needs contiguous tensors")
-    nbytes = src.numel() * src.element_size()
-    _require(nbytes == dst.numel() * dst.element_size(), "copy needs equally sized tensors")
-    with _on_device(dst):
-        _lib.check(_lib.lib().tw_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, _stream_ptr(dst)))
 
 
 def num_compute_units(device=None) -> int:

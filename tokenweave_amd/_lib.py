@@ -22,6 +22,8 @@ TW_DTYPE_BF16 = 0
 TW_DTYPE_F16 = 1
 TW_DTYPE_F32 = 2
 TW_MAX_PARTIALS = 16
+TW_SPLIT_MAX_TOKENS = 256
+TW_SPLIT_WORKSPACE_BYTES = TW_SPLIT_MAX_TOKENS * 384
 
 _vp, _i64, _u64, _f32, _ci = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_uint64,
                               ctypes.c_float, ctypes.c_int)
@@ -38,6 +40,10 @@ PROTOTYPES = {
     "tw_reduce_add_rms_norm": [ctypes.POINTER(_vp), _ci, _vp, _vp, _vp, _i64, _i64, _ci, _f32, _vp],
     "tw_fused_rs_ln_cta": [_vp, _vp, _vp, _u64, _i64, _ci, _ci, _ci, _f32, _i64, _i64, _vp],
     "tw_fused_rs_ln_ag_cta": [_vp, _vp, _vp, _u64, _i64, _ci, _ci, _ci, _f32, _i64, _i64, _vp],
+    "tw_reduce_add_rms_norm_ws": [ctypes.POINTER(_vp), _ci, _vp, _vp, _vp, _i64, _i64, _ci, _f32, _vp, _i64,
+                                  _vp],
+    "tw_fused_rs_ln_ag_cta_ws": [_vp, _vp, _vp, _u64, _i64, _ci, _ci, _ci, _f32, _i64, _i64, _vp, _i64, _vp],
+    "tw_split_segments": [_i64, _i64, _ci],
     "tw_gemm_bf16_nt": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp],
     "tw_rms_norm_static_fp8_quant": [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _ci, _vp],
     "tw_fused_add_rms_norm_static_fp8_quant": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _ci, _vp],
@@ -46,7 +52,6 @@ PROTOTYPES = {
     "tw_rms_norm_dynamic_per_token_quant": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _ci, _ci, _vp],
     "tw_reduce_add_rms_norm_dynamic_per_token_quant": [ctypes.POINTER(_vp), _ci, _vp, _vp, _vp, _vp, _vp,
                                                        _i64, _i64, _ci, _f32, _ci, _vp],
-    "tw_copy_bytes": [_vp, _vp, _i64, _vp],
 }
 
 _lib = None

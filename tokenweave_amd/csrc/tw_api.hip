@@ -19,6 +19,18 @@ int set_error(int code, const char* fmt, ...) {
   return code;
 }
 
+hipError_t& launch_status() {
+  static thread_local hipError_t status = hipSuccess;
+  return status;
+}
+
+int finish_launch(const char* what) {
+  const hipError_t e = launch_status();
+  if (e != hipSuccess)
+    return set_error(TW_ERR_LAUNCH, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
+  return TW_OK;
+}
+
 int device_compute_units() {
   constexpr int kMaxDevices = 64;
   static int cache[kMaxDevices];  // 0 = not queried yet
@@ -137,6 +149,43 @@ int tw_fused_rs_ln_ag_cta(void* input, void* residual, const void* weight, uint6
                           stream);
 }
 
+static int check_workspace(const char* what, const void* workspace, int64_t workspace_bytes) {
+  if (workspace && workspace_bytes < TW_SPLIT_WORKSPACE_BYTES)
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "%s: workspace of %lld bytes, need %d", what,
+                         (long long)workspace_bytes, TW_SPLIT_WORKSPACE_BYTES);
+  return TW_OK;
+}
+
+int tw_reduce_add_rms_norm_ws(const void* const* partials, int num_partials, void* y, void* residual,
+                              const void* weight, int64_t num_tokens, int64_t hidden_size,
+                              int max_ctas, float epsilon, void* workspace, int64_t workspace_bytes,
+                              void* stream) {
+  if (int rc = check_workspace("reduce_add_rms_norm_ws", workspace, workspace_bytes)) return rc;
+  if (!residual && num_tokens > 0)
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "reduce_add_rms_norm_ws: residual is null");
+  return tw::run_row_norm_ws("reduce_add_rms_norm_ws", partials, num_partials, y, residual, weight,
+                             num_tokens, hidden_size, epsilon, max_ctas, workspace, stream);
+}
+
+int tw_fused_rs_ln_ag_cta_ws(void* input, void* residual, const void* weight, uint64_t mcptr,
+                             int64_t peer_stride_bytes, int rank, int world_size, int max_ctas,
+                             float epsilon, int64_t num_tokens, int64_t hidden_size, void* workspace,
+                             int64_t workspace_bytes, void* stream) {
+  if (int rc = check_workspace("fused_rs_ln_ag_cta_ws", workspace, workspace_bytes)) return rc;
+  const void* parts[TW_MAX_PARTIALS];
+  int rc = tw::strided_partials("fused_rs_ln_ag_cta_ws", mcptr, peer_stride_bytes, rank, world_size,
+                                parts);
+  if (rc != TW_OK) return rc;
+  if (!residual && num_tokens > 0)
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "fused_rs_ln_ag_cta_ws: residual is null");
+  return tw::run_row_norm_ws("fused_rs_ln_ag_cta_ws", parts, world_size, input, residual, weight,
+                             num_tokens, hidden_size, epsilon, max_ctas, workspace, stream);
+}
+
+int tw_split_segments(int64_t num_tokens, int64_t hidden_size, int max_ctas) {
+  return tw::split_segments(num_tokens, hidden_size, max_ctas);
+}
+
 int tw_rms_norm_static_fp8_quant(void* out, const void* input, const void* weight,
                                  const float* scale, int64_t num_tokens, int64_t hidden_size,
                                  float epsilon, int dtype, void* stream) {
@@ -201,10 +250,6 @@ int tw_reduce_add_rms_norm_dynamic_per_token_quant(const void* const* partials, 
   return tw::run_row_norm_q("reduce_add_rms_norm_dynamic_per_token_quant", partials, num_partials, out,
                             residual, nullptr, weight, quant, scale_ub, scales, num_tokens,
                             hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true, stream);
-}
-
-int tw_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
-  return tw::run_copy16(dst, src, nbytes, stream);
 }
 
 int tw_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t N, int64_t K,

@@ -470,8 +470,8 @@ static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64
   if (max_cus > 0 && grid > max_cus) grid = max_cus;
   // 16-byte stores need 16-byte aligned row segments that end inside the row
   const int wide_store = (N % 8 == 0 && ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) ? 1 : 0;
-  hipLaunchKernelGGL((gemm_bf16_nt_big_kernel<TM, TN>), dim3((unsigned)grid), dim3(BIG_THREADS), LDS, hs,
-                     out, a, b, (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n, wide_store);
+  launch_kernel(gemm_bf16_nt_big_kernel<TM, TN>, dim3((unsigned)grid), dim3(BIG_THREADS), LDS, hs, out, a, b,
+                (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n, wide_store);
   return TW_OK;
 }
 
@@ -540,14 +540,11 @@ int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t
     int64_t grid = (int64_t)tiles_m * tiles_n;
     if (max_cus > 0 && grid > max_cus) grid = max_cus;
     if (grid > INT32_MAX) grid = INT32_MAX;
-    hipLaunchKernelGGL(gemm_bf16_nt_kernel, dim3((unsigned)grid), dim3(GEMM_THREADS), 0, hs,
-                       static_cast<uint16_t*>(out), static_cast<const uint16_t*>(a),
-                       static_cast<const uint16_t*>(b), (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n);
+    launch_kernel(gemm_bf16_nt_kernel, dim3((unsigned)grid), dim3(GEMM_THREADS), 0, hs,
+                  static_cast<uint16_t*>(out), static_cast<const uint16_t*>(a),
+                  static_cast<const uint16_t*>(b), (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n);
   }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess)
-    return set_error(TW_ERR_LAUNCH, "gemm_bf16_nt: kernel launch failed: %s", hipGetErrorString(e));
-  return TW_OK;
+  return finish_launch("gemm_bf16_nt");
 }
 
 }  // namespace tw

@@ -45,6 +45,36 @@ struct PartialPtrs {
   const void* p[TW_MAX_PARTIALS];
 };
 
+// Timeline stamps of the vector kernel.  They exist only in the measurement build of this
+// file (the benchmark's own library defines TW_TRACE before including it): per token
+// row, the constant-rate wall clock at a few program points and the hardware ids of
+// the compute unit, written by lane 0 to a buffer the benchmark supplies.  The drained
+// form first waits for the wave's outstanding memory operations.
+#ifdef TW_TRACE
+__device__ unsigned long long* g_trace;
+constexpr int kTraceSlots = 8;
+#define TW_STAMP(row, i)                                                                         \
+  do {                                                                                           \
+    if (threadIdx.x == 0) g_trace[(size_t)(row) * kTraceSlots + (i)] = wall_clock64();           \
+  } while (0)
+#define TW_STAMP_DRAINED(row, i)                                                                 \
+  do {                                                                                           \
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                             \
+    TW_STAMP(row, i);                                                                            \
+  } while (0)
+#define TW_STAMP_HWID(row, i)                                                                    \
+  do {                                                                                           \
+    if (threadIdx.x == 0)                                                                        \
+      g_trace[(size_t)(row) * kTraceSlots + (i)] =                                               \
+          ((unsigned long long)__builtin_amdgcn_s_getreg((4 - 1) << 11 | 20) << 32) |            \
+          (unsigned)__builtin_amdgcn_s_getreg((32 - 1) << 11 | 4);                               \
+  } while (0)
+#else
+#define TW_STAMP(row, i)
+#define TW_STAMP_DRAINED(row, i)
+#define TW_STAMP_HWID(row, i)
+#endif
+
 // ---------------------------------------------------------------------------
 // bf16 helpers.  A 32-bit word holds two bf16: element 2i in the low half.
 // ---------------------------------------------------------------------------
@@ -334,6 +364,9 @@ __device__ __forceinline__ void row_norm_vec_body(
   for (int row = blockIdx.x; row < num_tokens; row += gridDim.x, phase ^= 1) {
     float s[VPT][8];
     uint4 first[VPT];
+    uint4 wv[VPT];     // the weight row is fetched per token row, behind the row's own loads
+    TW_STAMP(row, 0);  // row begins
+    TW_STAMP_HWID(row, 6);
     const __amdgpu_buffer_rsrc_t dr = row_desc(HAS_RES ? residual : parts.p[0], row, row_bytes);
 
     if (NP > 0 && (VPT <= 2 || MAXNT <= 256)) {
@@ -352,13 +385,30 @@ __device__ __forceinline__ void row_norm_vec_body(
 #pragma unroll
         for (int k = 0; k < VPT; ++k) rv[k] = load16<kLoadStream>(dr, off[k]);
       }
+      // Nothing below may be scheduled above this point and no load of the row below
+      // it: the compiler would otherwise trade loads in flight for registers.
+      __builtin_amdgcn_sched_barrier(0);
+      // The weight row goes last: an L2 hit after the first workgroups, and its
+      // (cold) latency must not sit ahead of the row's own loads.  (Issued ahead of
+      // the barrier it costs the P = 1 op 8 % at 512 rows.)
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) wv[k] = load16<kLoadCached>(dw, off[k]);
+      // Accumulate stream by stream, in the order the loads were issued: the arithmetic
+      // on the first partials runs while the later ones are still on their way.  (Per
+      // element the order of the additions is p = 0 .. P-1, then the residual, either way.)
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
         first[k] = a[k][0];
         unpack8e<E>(a[k][0], s[k]);
+      }
 #pragma unroll
-        for (int p = 1; p < NP; ++p) add8e<E>(a[k][p], s[k]);
-        if (HAS_RES) add8e<E>(rv[k], s[k]);
+      for (int p = 1; p < NP; ++p) {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) add8e<E>(a[k][p], s[k]);
+      }
+      if (HAS_RES) {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) add8e<E>(rv[k], s[k]);
       }
     } else {
       {
@@ -378,14 +428,11 @@ __device__ __forceinline__ void row_norm_vec_body(
 #pragma unroll
         for (int k = 0; k < VPT; ++k) add8e<E>(load16<kLoadStream>(dr, off[k]), s[k]);
       }
-    }
-    // The weight row is fetched per token row, behind the row's own loads: it is
-    // an L2 hit after the first workgroups, and fetching it up front would put
-    // its (cold) latency ahead of the first partial load.
-    uint4 wv[VPT];
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) wv[k] = load16<kLoadCached>(dw, off[k]);
+      for (int k = 0; k < VPT; ++k) wv[k] = load16<kLoadCached>(dw, off[k]);
+    }
 
+    TW_STAMP_DRAINED(row, 1);  // every load of the row (and the weight) has returned
     if (COPY) {
       const __amdgpu_buffer_rsrc_t dc = row_desc(copy_out, row, row_bytes);
 #pragma unroll
@@ -408,8 +455,10 @@ __device__ __forceinline__ void row_norm_vec_body(
       if (HAS_RES) store16(dr, off[k], rnew[k]);
     }
 
+    TW_STAMP(row, 2);  // residual stores issued
     const float total = row_sum_chunks<VPT>(ss, slots[phase], nwaves, nchunks);
     const float inv = inv_rms(total, hidden, eps);
+    TW_STAMP(row, 3);  // row sum known
 
     // bf16 output: 16 bytes per vector; fp8 output: the bf16 result quantised, 8 bytes
     // per vector in rows of half the size.
@@ -472,6 +521,8 @@ __device__ __forceinline__ void row_norm_vec_body(
         store16(dy, off[k], o);
       }
     }
+    TW_STAMP(row, 4);          // y stores issued
+    TW_STAMP_DRAINED(row, 5);  // every store of the row acknowledged
   }
 }
 
@@ -498,6 +549,171 @@ __global__ __launch_bounds__(MAXNT) void row_norm_f16_kernel(
   row_norm_vec_body<_Float16, 1, VPT, MAXNT, HAS_RES, COPY, Q>(parts, 1, y_out, residual, copy_out, weight,
                                                              quant_scale, row_scales, eps, num_tokens,
                                                              vec_per_row, hidden, slots, max_slots);
+}
+
+// ---------------------------------------------------------------------------
+// Split rows: few token rows, many compute units (decode batches).
+//
+// A row is cut into `segs` segments of whole 64-vector chunks and every segment
+// gets its own workgroup, so one row's (P + 1) input streams are pulled by
+// several compute units at once.  A segment workgroup does the first half of the
+// row kernel on its vectors — fp32 sum, rounded residual stored, one sum of
+// squares per chunk by wave_sum — and leaves its chunk sums in the row's slot of
+// a small workspace.  It then counts itself in on the row's arrival counter.  The
+// workgroup that arrives last finds every chunk sum of the row there, reduces
+// them exactly as row_sum_chunks does (chunk c in lane c, one wave_sum), and
+// writes y for the WHOLE row from the rounded residual it re-reads — the same
+// operands in the same order as the one-workgroup kernel, hence the same bits.
+// Nobody waits for anybody: a workgroup that is not last is finished, so the
+// kernel makes progress whatever the dispatch order and needs no co-residency.
+//
+// Ordering: what one workgroup hands to another — the rounded residual and the
+// chunk sums — is written with device-scope stores (write-through past the XCD's L2,
+// so no L2 write-back is needed to publish them), every wave waits for its stores to
+// be acknowledged before the workgroup's arrival is counted (a device-scope atomic),
+// and the last workgroup reads them back with device-scope loads, which do not hit
+// in a per-compute-unit cache or another XCD's L2.  The last workgroup of a row
+// resets the row's counter, so the counters are zero again when the kernel ends;
+// calls that share a workspace must not overlap in time.
+//
+// Workgroup b serves row 8 (b / (8 segs)) + b % 8, segment (b / 8) % segs: the
+// segments of one row have equal b % 8 and so are dispatched to one XCD, whose L2
+// then holds the residual for the last workgroup's re-read.
+// ---------------------------------------------------------------------------
+struct SplitRow {
+  float sums[kMaxChunks];  // chunk sums of squares of the row in flight (two 128-byte lines)
+  uint32_t arrived;        // segment workgroups that have delivered theirs (a line of its own)
+  uint32_t pad[31];
+};
+static_assert(sizeof(SplitRow) * TW_SPLIT_MAX_TOKENS == TW_SPLIT_WORKSPACE_BYTES,
+              "workspace layout and the public size disagree");
+
+constexpr int kLoadDevice = 16;   // sc1: coherent at device scope
+constexpr int kStoreDevice = 16;  // sc1: written through to device scope
+
+__device__ __forceinline__ void store16_device(__amdgpu_buffer_rsrc_t d, uint32_t off, const uint4& v) {
+  u32x4_t t = {v.x, v.y, v.z, v.w};
+  __builtin_amdgcn_raw_buffer_store_b128(t, d, off, 0, kStoreDevice);
+}
+
+// XCD_ROWS: the segments of one row are workgroups with equal blockIdx % 8.
+template <int NP, int VPT, bool XCD_ROWS>
+__global__ __launch_bounds__(1024) void row_norm_split_kernel(
+    PartialPtrs parts, int np_rt, void* y_out, void* residual, const void* __restrict__ weight,
+    SplitRow* __restrict__ ws, float eps, int num_tokens, int vec_per_row, float hidden, int segs) {
+  __shared__ uint32_t arrivals_before;
+  const int nt = blockDim.x;
+  const int nwaves = nt >> 6;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int nchunks = (vec_per_row + 63) >> 6;
+  const int np = NP > 0 ? NP : np_rt;
+  const uint32_t row_bytes = (uint32_t)vec_per_row * 16u;
+
+  const int per_group = 8 * segs;
+  const int row = XCD_ROWS ? (blockIdx.x / per_group) * 8 + (blockIdx.x & 7) : blockIdx.x / segs;
+  const int seg = XCD_ROWS ? (blockIdx.x % per_group) >> 3 : blockIdx.x % segs;
+  if (row >= num_tokens) return;
+  const int chunk0 = seg * VPT * nwaves;  // first chunk of this segment
+
+  uint32_t off[VPT];
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) off[k] = (uint32_t)((chunk0 + k * nwaves) * 64 + (int)threadIdx.x) * 16u;
+
+  const __amdgpu_buffer_rsrc_t dr = row_desc(residual, row, row_bytes);
+  float s[VPT][8];
+  if (NP > 0) {
+    uint4 a[VPT][NP > 0 ? NP : 1];
+    uint4 rv[VPT];
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[p], row, row_bytes);
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) a[k][p] = load16<kLoadStream>(dp, off[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) rv[k] = load16<kLoadStream>(dr, off[k]);
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) unpack8(a[k][0], s[k]);
+#pragma unroll
+    for (int p = 1; p < NP; ++p) {
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) add8(a[k][p], s[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) add8(rv[k], s[k]);
+  } else {
+    {
+      const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[0], row, row_bytes);
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) unpack8(load16<kLoadStream>(dp, off[k]), s[k]);
+    }
+    for (int p = 1; p < np; ++p) {
+      const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[p], row, row_bytes);
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dp, off[k]), s[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dr, off[k]), s[k]);
+  }
+
+  SplitRow* slot = ws + row;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    float ss = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += s[k][e] * s[k][e];
+    uint4 rnew;
+    rnew.x = pack_bf16(s[k][0], s[k][1]);
+    rnew.y = pack_bf16(s[k][2], s[k][3]);
+    rnew.z = pack_bf16(s[k][4], s[k][5]);
+    rnew.w = pack_bf16(s[k][6], s[k][7]);
+    store16_device(dr, off[k], rnew);
+    const float c = wave_sum(ss);
+    const int chunk = chunk0 + k * nwaves + wave;
+    if (lane == 0 && chunk < nchunks)
+      __hip_atomic_store(&slot->sums[chunk], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  // every store of this wave has been acknowledged at device scope before the
+  // workgroup's arrival is counted
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0)
+    arrivals_before = __hip_atomic_fetch_add(&slot->arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (arrivals_before != (uint32_t)(segs - 1)) return;
+
+  // Last workgroup of the row: all chunk sums are in the slot.
+  if (threadIdx.x == 0) __hip_atomic_store(&slot->arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const float cs = lane < nchunks
+                       ? __hip_atomic_load(&slot->sums[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                       : 0.0f;
+  const float inv = inv_rms(wave_sum(cs), hidden, eps);
+
+  const __amdgpu_buffer_rsrc_t dw = row_desc(weight, 0, row_bytes);
+  const __amdgpu_buffer_rsrc_t dy = row_desc(y_out, row, row_bytes);
+  constexpr int U = 4;  // vectors in flight per lane
+  for (int v0 = threadIdx.x; v0 < vec_per_row; v0 += U * nt) {
+    uint4 rv[U], wv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t o = (uint32_t)(v0 + u * nt) * 16u;  // past the row's end: zeros, store dropped
+      rv[u] = load16<kLoadDevice>(dr, o);
+      wv[u] = load16<kLoadCached>(dw, o);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float r[8], w[8];
+      unpack8(rv[u], r);
+      unpack8(wv[u], w);
+      uint4 o;
+      o.x = pack_bf16(r[0] * inv * w[0], r[1] * inv * w[1]);
+      o.y = pack_bf16(r[2] * inv * w[2], r[3] * inv * w[3]);
+      o.z = pack_bf16(r[4] * inv * w[4], r[5] * inv * w[5]);
+      o.w = pack_bf16(r[6] * inv * w[6], r[7] * inv * w[7]);
+      store16(dy, (uint32_t)(v0 + u * nt) * 16u, o);
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -675,6 +891,7 @@ struct RowNormArgs {
   int q;                     // output kind (kQNone ..)
   const float* quant_scale;  // static fp8: the scale; dynamic fp8: optional upper bound (may be null)
   float* row_scales;         // dynamic kinds: one scale per row (output)
+  SplitRow* split_ws;        // workspace of the split-row kernel, or null
   int64_t T, H;
   float eps;
   int grid;
@@ -691,7 +908,7 @@ static int launch_vec(const RowNormArgs& a) {
   if (a.f16) {
     if (NP != 1) return 1;
 #define TW_LAUNCH_F16(VPT, MAXNT)                                                                \
-  hipLaunchKernelGGL((row_norm_f16_kernel<VPT, MAXNT, HAS_RES, COPY, Q>), g, b, 0, a.stream,     \
+  launch_kernel(row_norm_f16_kernel<VPT, MAXNT, HAS_RES, COPY, Q>, g, b, 0, a.stream,            \
                      a.parts, a.y, a.residual, a.copy_out, a.weight, a.quant_scale,              \
                      a.row_scales, a.eps, (int)a.T, V, (float)a.H)
     if (sh.vpt == 1) TW_LAUNCH_F16(1, 1024);
@@ -702,7 +919,7 @@ static int launch_vec(const RowNormArgs& a) {
     return 0;
   }
 #define TW_LAUNCH(VPT, MAXNT)                                                                    \
-  hipLaunchKernelGGL((row_norm_bf16_kernel<NP, VPT, MAXNT, HAS_RES, COPY, Q>), g, b, 0,          \
+  launch_kernel(row_norm_bf16_kernel<NP, VPT, MAXNT, HAS_RES, COPY, Q>, g, b, 0,                 \
                      a.stream, a.parts, a.np, a.y, a.residual, a.copy_out, a.weight,             \
                      a.quant_scale, a.row_scales, a.eps, (int)a.T, V, (float)a.H)
   if (sh.vpt == 1) TW_LAUNCH(1, 1024);
@@ -711,6 +928,58 @@ static int launch_vec(const RowNormArgs& a) {
   else TW_LAUNCH(4, 1024);
 #undef TW_LAUNCH
   return 0;
+}
+
+// The split-row kernel exists for the fused op proper: bf16 vector rows, residual
+// add, bf16 output.
+static bool splittable(bool vec_ok, int dtype, const void* residual, const void* copy_out, int quant) {
+  return vec_ok && dtype == TW_DTYPE_BF16 && residual && !copy_out && quant == kQNone;
+}
+
+// Segments per row and workgroup shape of the split-row kernel, or false when the
+// one-workgroup-per-row kernel is the better (or only) choice.  A segment is
+// vpt * nwaves whole chunks.
+struct SplitPlan { int vpt, nwaves, segs; };
+
+static bool split_plan(int V, int64_t T, int cus, SplitPlan* sp) {
+  const int nchunks = (V + 63) / 64;
+  if (T < 1 || T > TW_SPLIT_MAX_TOKENS || nchunks < 2 || nchunks > kMaxChunks || cus <= 0) return false;
+  // Measured with cold operands at hidden sizes 4096 .. 16384 and 1 .. 128 rows, over
+  // segments of 1 .. 16 chunks with 1, 2 or 4 vectors per lane: segments of four chunks
+  // with one vector per lane (256 lanes) are the fastest split; they beat one workgroup
+  // per row by 0.3 - 0.8 us at hidden size 8192 and by 2 - 3 us at 16384 up to 48 rows,
+  // draw level at 64 rows, and lose at 128 rows and for rows shorter than 16 chunks (the
+  // hand-over costs more than the shorter load phase saves).  Eight-chunk segments take
+  // over when four-chunk ones would make more workgroups than there are compute units.
+  if (T > 48 || nchunks < 16) return false;
+  sp->vpt = 1;
+  sp->nwaves = T * ((nchunks + 3) / 4) <= cus ? 4 : 8;
+  sp->segs = (nchunks + sp->nwaves - 1) / sp->nwaves;
+  return sp->segs >= 2;
+}
+
+template <int NP>
+static void launch_split(const RowNormArgs& a, const SplitPlan& sp) {
+  const int V = (int)(a.H / 8);
+  const int groups = (int)((a.T + 7) / 8);
+  dim3 g((unsigned)(groups * 8 * sp.segs)), b((unsigned)(sp.nwaves * 64));
+#define TW_LAUNCH_SPLIT(VPT)                                                                     \
+  launch_kernel(row_norm_split_kernel<NP, VPT, true>, g, b, 0, a.stream, a.parts, a.np, a.y,     \
+                a.residual, a.weight, a.split_ws, a.eps, (int)a.T, V, (float)a.H, sp.segs)
+  if (sp.vpt == 1) TW_LAUNCH_SPLIT(1);
+  else if (sp.vpt == 2) TW_LAUNCH_SPLIT(2);
+  else TW_LAUNCH_SPLIT(4);
+#undef TW_LAUNCH_SPLIT
+}
+
+static void launch_split_np(const RowNormArgs& a, const SplitPlan& sp) {
+  switch (a.np) {
+    case 1: launch_split<1>(a, sp); break;
+    case 2: launch_split<2>(a, sp); break;
+    case 4: launch_split<4>(a, sp); break;
+    case 8: launch_split<8>(a, sp); break;
+    default: launch_split<0>(a, sp); break;
+  }
 }
 
 // mode: residual given -> add + write back; copy_out given -> rms_norm_inplace;
@@ -742,12 +1011,12 @@ static void launch_elem(const RowNormArgs& a) {
   int nt = a.H < 1024 ? (int)((a.H + 63) / 64) * 64 : 1024;
   dim3 g(a.grid), b(nt);
 #define TW_LAUNCH(HAS_RES, COPY, FP8)                                                            \
-  hipLaunchKernelGGL((row_norm_elem_kernel<T, HAS_RES, COPY, FP8>), g, b, 0, a.stream, a.parts,  \
+  launch_kernel(row_norm_elem_kernel<T, HAS_RES, COPY, FP8>, g, b, 0, a.stream, a.parts,         \
                      a.np, a.y, static_cast<T*>(a.residual), static_cast<T*>(a.copy_out),        \
                      static_cast<const T*>(a.weight), a.quant_scale, a.eps, (int)a.T, (int)a.H)
   if (a.q == kQDynFp8 || a.q == kQDynInt8) {
 #define TW_LAUNCH_DYN(HAS_RES, INT8)                                                             \
-  hipLaunchKernelGGL((row_norm_dyn_elem_kernel<T, HAS_RES, INT8>), g, b, 0, a.stream, a.parts,   \
+  launch_kernel(row_norm_dyn_elem_kernel<T, HAS_RES, INT8>, g, b, 0, a.stream, a.parts,          \
                      a.np, static_cast<uint8_t*>(a.y), a.row_scales, static_cast<T*>(a.residual), \
                      static_cast<const T*>(a.weight), a.quant_scale, a.eps, (int)a.T, (int)a.H)
     if (a.residual) { if (a.q == kQDynInt8) TW_LAUNCH_DYN(true, true); else TW_LAUNCH_DYN(true, false); }
@@ -762,23 +1031,17 @@ static void launch_elem(const RowNormArgs& a) {
 #undef TW_LAUNCH
 }
 
-static int finish_launch(const char* what) {
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess)
-    return set_error(TW_ERR_LAUNCH, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
-  return TW_OK;
-}
-
 // Shared by every entry point.  residual == nullptr: no residual add;
 // copy_out != nullptr: rms_norm_inplace; quant: 0 = y in the input's type, 1 = fp8
 // with the static scale *quant_scale, 2 / 3 = dynamic per-token fp8 / int8 (row scales
 // to row_scales, quant_scale = optional upper bound).
 // require_vec: refuse instead of falling back to the element-wise kernel (the
 // *_cta contract).
-int run_row_norm_q(const char* what, const void* const* partials, int np, void* y,
-                   void* residual, void* copy_out, const void* weight, int quant,
-                   const float* quant_scale, float* row_scales, int64_t T, int64_t H, float eps,
-                   int dtype, int max_ctas, bool require_vec, void* stream_v) {
+static int run_row_norm_any(const char* what, const void* const* partials, int np, void* y,
+                            void* residual, void* copy_out, const void* weight, int quant,
+                            const float* quant_scale, float* row_scales, int64_t T, int64_t H, float eps,
+                            int dtype, int max_ctas, bool require_vec, void* split_workspace,
+                            void* stream_v) {
   if (np < 1 || np > TW_MAX_PARTIALS)
     return set_error(TW_ERR_INVALID_ARGUMENT, "%s: number of partials %d not in [1, %d]", what, np,
                      TW_MAX_PARTIALS);
@@ -835,6 +1098,17 @@ int run_row_norm_q(const char* what, const void* const* partials, int np, void* 
   a.grid = grid;
   a.stream = static_cast<hipStream_t>(stream_v);
 
+  // Few rows and a workspace: several workgroups per row.  A grid cap is a compute-unit
+  // budget and is honoured by not splitting.
+  if (split_workspace && max_ctas <= 0 && splittable(vec_ok, dtype, residual, copy_out, quant)) {
+    SplitPlan sp;
+    if (split_plan((int)(H / 8), T, device_compute_units(), &sp)) {
+      a.split_ws = static_cast<SplitRow*>(split_workspace);
+      launch_split_np(a, sp);
+      return finish_launch(what);
+    }
+  }
+
   if (vec_ok && (dtype == TW_DTYPE_BF16 || (dtype == TW_DTYPE_F16 && np == 1))) {
     int fell = 1;
     switch (np) {
@@ -856,6 +1130,29 @@ int run_row_norm_q(const char* what, const void* const* partials, int np, void* 
   return finish_launch(what);
 }
 
+int run_row_norm_q(const char* what, const void* const* partials, int np, void* y,
+                   void* residual, void* copy_out, const void* weight, int quant,
+                   const float* quant_scale, float* row_scales, int64_t T, int64_t H, float eps,
+                   int dtype, int max_ctas, bool require_vec, void* stream) {
+  return run_row_norm_any(what, partials, np, y, residual, copy_out, weight, quant, quant_scale, row_scales,
+                          T, H, eps, dtype, max_ctas, require_vec, nullptr, stream);
+}
+
+int run_row_norm_ws(const char* what, const void* const* partials, int np, void* y, void* residual,
+                    const void* weight, int64_t T, int64_t H, float eps, int max_ctas,
+                    void* workspace, void* stream) {
+  if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return set_error(TW_ERR_ALIGNMENT, "%s: the workspace must be 256-byte aligned", what);
+  return run_row_norm_any(what, partials, np, y, residual, nullptr, weight, kQNone, nullptr, nullptr, T, H,
+                          eps, TW_DTYPE_BF16, max_ctas, true, workspace, stream);
+}
+
+int split_segments(int64_t T, int64_t H, int max_ctas) {
+  SplitPlan sp;
+  if (max_ctas > 0 || H <= 0 || H % 8 != 0 || H / 8 > INT32_MAX) return 1;
+  return split_plan((int)(H / 8), T, device_compute_units(), &sp) ? sp.segs : 1;
+}
+
 int run_row_norm(const char* what, const void* const* partials, int np, void* y,
                  void* residual, void* copy_out, const void* weight, const float* quant_scale,
                  int64_t T, int64_t H, float eps, int dtype, int max_ctas, bool require_vec,
@@ -863,37 +1160,6 @@ int run_row_norm(const char* what, const void* const* partials, int np, void* y,
   return run_row_norm_q(what, partials, np, y, residual, copy_out, weight,
                         quant_scale ? kQStaticFp8 : kQNone, quant_scale, nullptr, T, H, eps, dtype,
                         max_ctas, require_vec, stream);
-}
-
-// ---------------------------------------------------------------------------
-// Plain copy with default cache policy: the known-size traffic against which
-// hardware memory counters are scaled.
-// ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void copy16_kernel(uint4* __restrict__ dst,
-                                                     const uint4* __restrict__ src, size_t n) {
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
-}
-
-int run_copy16(void* dst, const void* src, int64_t nbytes, void* stream) {
-  if (nbytes < 0 || nbytes % 16 != 0)
-    return set_error(TW_ERR_INVALID_ARGUMENT, "copy: byte count %lld is not a non-negative multiple of 16",
-                     (long long)nbytes);
-  if (nbytes == 0) return TW_OK;
-  if (!dst || !src) return set_error(TW_ERR_INVALID_ARGUMENT, "copy: null pointer argument");
-  if ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u)
-    return set_error(TW_ERR_ALIGNMENT, "copy: pointers must be 16-byte aligned");
-  const size_t n = (size_t)nbytes / 16;
-  const int cus = device_compute_units();
-  size_t blocks = (n + 255) / 256;
-  const size_t cap = (size_t)(cus > 0 ? cus : 256) * 16;
-  if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<uint4*>(dst), static_cast<const uint4*>(src), n);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess)
-    return set_error(TW_ERR_LAUNCH, "copy: kernel launch failed: %s", hipGetErrorString(e));
-  return TW_OK;
 }
 
 }  // namespace tw

@@ -101,7 +101,7 @@ class PartialsBuffer:
         self.multicast_ptr = self._backing.data_ptr()
         self.signal_pad_ptrs_dev = 0
         ops.register_partials_region(self.multicast_ptr, self.peer_stride_bytes, world_size,
-                                     self._backing)
+                                     self._backing, usable_bytes=max_tokens * hidden_size * 2)
 
     def slot(self, p: int) -> torch.Tensor:
         """Rank p's staging buffer, [max_tokens, hidden_size]."""

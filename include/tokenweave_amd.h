@@ -171,6 +171,23 @@ TW_API int tw_fused_rs_ln_ag_cta_ws(void* input, void* residual, const void* wei
                              void* workspace, int64_t workspace_bytes,
                              void* stream);
 
+/* tw_reduce_add_rms_norm_ws without a workspace argument and without any
+ * allocation: the workspace is a static array in the library's device code
+ * (TW_SPLIT_WORKSPACE_BYTES = 96 KiB on every GPU the library is used on, held
+ * until the process ends).  No counterpart in the reference; it is for callers
+ * that cannot allocate device memory — code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  num_tokens above
+ * TW_SPLIT_MAX_TOKENS is refused with TW_ERR_INVALID_ARGUMENT (such batches need
+ * no workspace: use tw_reduce_add_rms_norm).  The first call on a device resolves
+ * the array's address (not a stream operation: make it before capturing).  All
+ * calls on one GPU share the one array: calls that overlap in time on the same GPU
+ * (different streams, no ordering) race; order them or use the *_ws form with a
+ * workspace per stream. */
+TW_API int tw_reduce_add_rms_norm_noalloc(const void* const* partials, int num_partials,
+                                   void* y, void* residual, const void* weight,
+                                   int64_t num_tokens, int64_t hidden_size,
+                                   int max_ctas, float epsilon, void* stream);
+
 /* Segments per row the *_ws entry points use for this shape on the current
  * device: 1 = one workgroup per row (no workspace traffic). */
 TW_API int tw_split_segments(int64_t num_tokens, int64_t hidden_size, int max_ctas);

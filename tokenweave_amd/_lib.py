@@ -43,6 +43,7 @@ PROTOTYPES = {
     "tw_reduce_add_rms_norm_ws": [ctypes.POINTER(_vp), _ci, _vp, _vp, _vp, _i64, _i64, _ci, _f32, _vp, _i64,
                                   _vp],
     "tw_fused_rs_ln_ag_cta_ws": [_vp, _vp, _vp, _u64, _i64, _ci, _ci, _ci, _f32, _i64, _i64, _vp, _i64, _vp],
+    "tw_reduce_add_rms_norm_noalloc": [ctypes.POINTER(_vp), _ci, _vp, _vp, _vp, _i64, _i64, _ci, _f32, _vp],
     "tw_split_segments": [_i64, _i64, _ci],
     "tw_gemm_bf16_nt": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp],
     "tw_rms_norm_static_fp8_quant": [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _ci, _vp],

@@ -182,6 +182,15 @@ int tw_fused_rs_ln_ag_cta_ws(void* input, void* residual, const void* weight, ui
                              num_tokens, hidden_size, epsilon, max_ctas, workspace, stream);
 }
 
+int tw_reduce_add_rms_norm_noalloc(const void* const* partials, int num_partials, void* y, void* residual,
+                                   const void* weight, int64_t num_tokens, int64_t hidden_size,
+                                   int max_ctas, float epsilon, void* stream) {
+  if (!residual && num_tokens > 0)
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "reduce_add_rms_norm_noalloc: residual is null");
+  return tw::run_row_norm_noalloc("reduce_add_rms_norm_noalloc", partials, num_partials, y, residual, weight,
+                                  num_tokens, hidden_size, epsilon, max_ctas, stream);
+}
+
 int tw_split_segments(int64_t num_tokens, int64_t hidden_size, int max_ctas) {
   return tw::split_segments(num_tokens, hidden_size, max_ctas);
 }

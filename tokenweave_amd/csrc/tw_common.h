@@ -59,6 +59,10 @@ int run_row_norm_ws(const char* what, const void* const* partials, int np, void*
                     const void* weight, int64_t T, int64_t H, float eps, int max_ctas,
                     void* workspace, void* stream);
 
+// run_row_norm_ws on the library's static workspace; refuses T > TW_SPLIT_MAX_TOKENS.
+int run_row_norm_noalloc(const char* what, const void* const* partials, int np, void* y, void* residual,
+                         const void* weight, int64_t T, int64_t H, float eps, int max_ctas, void* stream);
+
 // Segments per row the split-row kernel would use for this shape on the current device
 // (1 = the one-workgroup-per-row kernel runs instead).
 int split_segments(int64_t T, int64_t H, int max_ctas);

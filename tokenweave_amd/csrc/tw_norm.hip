@@ -34,6 +34,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "tw_common.h"
 
 namespace tw {
@@ -1145,6 +1147,49 @@ int run_row_norm_ws(const char* what, const void* const* partials, int np, void*
     return set_error(TW_ERR_ALIGNMENT, "%s: the workspace must be 256-byte aligned", what);
   return run_row_norm_any(what, partials, np, y, residual, nullptr, weight, kQNone, nullptr, nullptr, T, H,
                           eps, TW_DTYPE_BF16, max_ctas, true, workspace, stream);
+}
+
+// ---------------------------------------------------------------------------
+// The split-row workspace as a static device array, for callers that cannot
+// allocate.  Every GPU the library runs on holds its own copy at its own address
+// until the process ends; the address is resolved once per device, with that
+// device current, and the kernels receive it as an argument exactly as they
+// receive a caller's workspace.  The array is zero when the code object is loaded
+// and every call's kernel leaves the arrival counters zero again, which is all that
+// must be zero at the start of a call; the chunk sums are rewritten before they are
+// read.  All calls on one GPU share the array: calls that overlap in time race.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[TW_SPLIT_WORKSPACE_BYTES];
+
+static int static_scratch(const char* what, void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<void*> resolved[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return set_error(TW_ERR_LAUNCH, "%s: no current device", what);
+  void* ptr = resolved[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return set_error(TW_ERR_LAUNCH, "%s: could not resolve the static workspace on device %d: %s", what, dev,
+                       hipGetErrorString(e));
+    resolved[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return TW_OK;
+}
+
+int run_row_norm_noalloc(const char* what, const void* const* partials, int np, void* y, void* residual,
+                         const void* weight, int64_t T, int64_t H, float eps, int max_ctas, void* stream) {
+  if (T > TW_SPLIT_MAX_TOKENS)
+    return set_error(TW_ERR_INVALID_ARGUMENT,
+                     "%s: num_tokens %lld exceeds the %d rows the static workspace holds "
+                     "(larger batches need no workspace: call tw_reduce_add_rms_norm)",
+                     what, (long long)T, TW_SPLIT_MAX_TOKENS);
+  void* ws = nullptr;
+  if (int rc = static_scratch(what, &ws)) return rc;
+  return run_row_norm_any(what, partials, np, y, residual, nullptr, weight, kQNone, nullptr, nullptr, T, H,
+                          eps, TW_DTYPE_BF16, max_ctas, true, ws, stream);
 }
 
 int split_segments(int64_t T, int64_t H, int max_ctas) {

@@ -20,8 +20,9 @@ Fields beyond the usual ones:
   cpu_baseline  the CPU checker (oracle/, a port of the reference's
                 csrc/cpu/layernorm.cpp extended to P partials) timed on this box's
                 host cores on the same workload, for context only.
-  sweep         (--sweep) µs/call and GB/s of every benchmark configuration, and the
-                weave configuration's overlap figures.
+  weave         config 5: GEMM of one token split (all eight partial sums, and one rank's)
+                overlapped with the fused norm of the other split: alone, serial, overlapped.
+  sweep         (--sweep) µs/call and GB/s of every benchmark configuration.
 """
 import argparse
 import ctypes
@@ -92,6 +93,7 @@ def parse_args():
     ap.add_argument("--max-ctas", type=int, default=0, help="grid cap (0 = library default)")
     ap.add_argument("--sweep", action="store_true", help="also time every configuration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-weave", action="store_true", help="leave the config 5 weave block out of the line")
     ap.add_argument("--weave-only", action="store_true",
                     help="time only the GEMM + norm weave of config 5 and print its figures (for profiling)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -498,49 +500,72 @@ def cpu_baseline(cfg, budget_s):
                       f"median {med * 1e6:.0f} us/call, OpenMP over rows with {threads} threads"}
 
 
-def time_weave(device, norm_cap, gemm_cap, steps=200):
-    """Config 5: the bf16 MFMA GEMM of the 2458-row split (current stream) overlapped
-    with the fused norm of the 1638-row split (second stream).  Every figure is the
-    mean over `steps` back-to-back stages bracketed by HIP events; the norm inputs
-    rotate through 8 sets (2.4 GB) so it reads cold HBM.  Calls are pre-bound ctypes
-    calls (arguments validated once by the public shims) so that the host can enqueue
-    a stage faster than the GPU runs it."""
+_WEAVE_STREAMS = None
+
+
+def weave_streams():
+    """The two streams of every weave measurement, created once: HIP spreads streams over a
+    few hardware queues (4 by default) in creation order, and two streams that land on one
+    queue run their kernels one after the other."""
+    global _WEAVE_STREAMS
+    if _WEAVE_STREAMS is None:
+        import torch
+        _WEAVE_STREAMS = (torch.cuda.Stream(), torch.cuda.Stream())
+    return _WEAVE_STREAMS
+
+
+def time_weave(device, form="eight_partials", gemm_caps=(128,), norm_cap=0, steps=200):
+    """Config 5: the bf16 MFMA GEMM of the 2458-row split on the current stream overlapped with
+    the fused norm of the 1638-row split on a second stream.  form "eight_partials": the
+    producer of all P = 8 row-parallel partial sums of the split (one launch,
+    tw_gemm_bf16_nt_partials, into the 8 staging slots); "one_partial": one rank's GEMM.
+    Every figure is the mean over `steps` back-to-back stages bracketed by HIP events; the
+    norm inputs rotate through 8 sets (2.4 GB) so it reads cold HBM, the GEMM outputs through
+    as many staging buffers.  Calls are pre-bound (arguments validated once by the public
+    shims) so that the host enqueues a stage faster than the GPU runs it.  The overlapped
+    stage is timed for every GEMM compute-unit budget in `gemm_caps`; the best is reported."""
     import torch
     from tokenweave_amd import _custom_ops as ops
     from tokenweave_amd import workloads as wl
-    cfg, R = wl.C5_NORM, 8
-    inps = [wl.make_norm_inputs(cfg, device, seed_offset=i) for i in range(R)]
-    g = wl.make_gemm_inputs(device=device)
-    Ta, K = g.a.shape
-    N = g.b.shape[0]
-    stages = [torch.zeros((Ta, N), dtype=torch.bfloat16, device=device) for _ in range(R)]
-    main_s, side_s = torch.cuda.Stream(), torch.cuda.Stream()
-    gemms, norms = {}, {}
-    for cap in {0, gemm_cap}:
-        gemms[cap] = [ops.bind_gemm_bf16_nt(stages[i], g.a, g.b, cap or None) for i in range(R)]
-    for cap in {0, norm_cap}:
-        norms[cap] = [ops.bind_reduce_add_rms_norm(inp.partials, inp.partials[0], inp.residual, inp.weight,
-                                                   cfg.eps, cap or None) for inp in inps]
-    pm, ps = main_s, side_s
+    cfg = wl.C5_NORM
+    P = 8 if form == "eight_partials" else 1
+    R = 4 if P == 8 else 8
+    inps = [wl.make_norm_inputs(cfg, device, seed_offset=i) for i in range(8)]
+    gs = wl.make_partials_gemm_inputs(P, device=device)
+    Ta, K = gs[0].a.shape
+    N = gs[0].b.shape[0]
+    stages = [torch.zeros((P, Ta, N), dtype=torch.bfloat16, device=device) for _ in range(R)]
+    main_s, side_s = weave_streams()
+
+    def bind_gemm(i, cap):
+        if P == 1:
+            return ops.bind_gemm_bf16_nt(stages[i][0], gs[0].a, gs[0].b, cap or None)
+        return ops.bind_gemm_bf16_nt_partials([stages[i][p] for p in range(P)], [g.a for g in gs],
+                                              [g.b for g in gs], cap or None)
+    gemms = {cap: [bind_gemm(i, cap) for i in range(R)] for cap in {0, *gemm_caps}}
+    norms = {cap: [ops.bind_reduce_add_rms_norm(inp.partials, inp.partials[0], inp.residual, inp.weight,
+                                                cfg.eps, cap or None) for inp in inps] for cap in {0, norm_cap}}
 
     def gemm(i, cap, stream):
         gemms[cap][i % R](stream)
 
     def norm(i, cap, stream):
-        norms[cap][i % R](stream)
+        norms[cap][i % 8](stream)
 
-    def weave(i):
-        before = torch.cuda.Event()
-        before.record(main_s)
-        gemm(i, gemm_cap, pm)                 # GEMM first: it takes its CU budget ...
-        side_s.wait_event(before)
-        norm(i, norm_cap, ps)                 # ... and the norm fills the remaining CUs
-        main_s.wait_stream(side_s)
+    def weave(cap):
+        def stage(i):
+            before = torch.cuda.Event()
+            before.record(main_s)
+            gemm(i, cap, main_s)                  # GEMM first: it takes its CU budget ...
+            side_s.wait_event(before)
+            norm(i, norm_cap, side_s)             # ... and the norm fills the remaining CUs
+            main_s.wait_stream(side_s)
+        return stage
 
     def timed(step):
         torch.cuda.synchronize()
         with torch.cuda.stream(main_s):
-            for i in range(10):
+            for i in range(5):
                 step(i)
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -551,19 +576,37 @@ def time_weave(device, norm_cap, gemm_cap, steps=200):
             torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e3 / steps
 
-    t_a = timed(lambda i: gemm(i, 0, pm))
-    t_b = timed(lambda i: norm(i, 0, pm))
-    t_ser = timed(lambda i: (gemm(i, 0, pm), norm(i, 0, pm)))
-    t_ovl = timed(weave)
-    flops = 2.0 * Ta * N * K
-    return {"gemm_us": t_a, "norm_us": t_b, "serial_us": t_ser, "overlap_us": t_ovl,
-            "speedup": t_ser / t_ovl, "overlap_eff": (t_ser - t_ovl) / min(t_a, t_b),
-            "gemm_tflops_alone": flops / t_a / 1e6,
-            "gemm_mfma_util_alone": flops / t_a / 1e6 / MFMA_BF16_PEAK_TFLOPS,
-            "gemm_tflops_overlapped": flops / t_ovl / 1e6,
-            "gemm_mfma_util_overlapped": flops / t_ovl / 1e6 / MFMA_BF16_PEAK_TFLOPS,
-            "norm_gbps_alone": cfg.bytes / t_b / 1e3, "norm_gbps_overlapped": cfg.bytes / t_ovl / 1e3,
-            "norm_cap": norm_cap, "gemm_cap": gemm_cap}
+    t_a = timed(lambda i: gemm(i, 0, main_s))
+    t_b = timed(lambda i: norm(i, 0, main_s))
+    t_ser = timed(lambda i: (gemm(i, 0, main_s), norm(i, 0, main_s)))
+    by_cap = {cap: timed(weave(cap)) for cap in gemm_caps}
+    best_cap = min(by_cap, key=by_cap.get)
+    t_ovl = by_cap[best_cap]
+    flops = 2.0 * P * Ta * N * K
+    out = {"form": form, "gemm_us": t_a, "norm_us": t_b, "serial_us": t_ser, "overlap_us": t_ovl,
+           "speedup": t_ser / t_ovl, "overlap_eff": (t_ser - t_ovl) / min(t_a, t_b),
+           "gemm_tflops_alone": flops / t_a / 1e6,
+           "gemm_mfma_util_alone": flops / t_a / 1e6 / MFMA_BF16_PEAK_TFLOPS,
+           "gemm_mfma_util_in_stage": flops / t_ovl / 1e6 / MFMA_BF16_PEAK_TFLOPS,
+           "norm_gbps_alone": cfg.bytes / t_b / 1e3, "norm_gbps_in_stage": cfg.bytes / t_ovl / 1e3,
+           "norm_cap": norm_cap, "gemm_cus": best_cap, "stages_timed": steps,
+           "overlap_us_by_gemm_cus": {str(c): round(v, 2) for c, v in by_cap.items()}}
+    del gemms, norms, stages, inps, gs
+    torch.cuda.empty_cache()
+    return {k: (round(v, 4) if isinstance(v, float) else v) for k, v in out.items()}
+
+
+def weave_block(device, steps):
+    """Both forms of config 5 for the JSON line."""
+    caps = (128, 160, 192, 224, 240)
+    return {"workload": "c5 token weave: GEMM [2458, 1024] x [8192, 1024]^T of one split || fused P=8 norm of "
+                        "the 1638-row split, H=8192",
+            "definitions": "serial = both kernels on one stream; overlap = GEMM capped to gemm_cus compute "
+                           "units on the current stream, norm on a second stream; speedup = serial/overlap; "
+                           "overlap_eff = (serial - overlap)/min(gemm, norm); MFMA utilisation against "
+                           "2.5 PFLOP/s dense bf16",
+            "eight_partials": time_weave(device, "eight_partials", caps, steps=steps),
+            "one_partial": time_weave(device, "one_partial", caps, steps=steps)}
 
 
 def main():
@@ -589,9 +632,7 @@ def main():
               flush=True)
         return
     if args.weave_only:
-        w = time_weave(device, norm_cap=0, gemm_cap=128, steps=args.steps)
-        print(json.dumps({"c5_weave": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}}),
-              flush=True)
+        print(json.dumps({"weave": weave_block(device, min(args.steps, 200))}), flush=True)
         return
     log(f"[bench] {torch.cuda.get_device_name(0)}; workload {cfg.name}: P={cfg.P} T={cfg.T} "
         f"H={cfg.H} bytes/call={cfg.bytes}")
@@ -628,6 +669,9 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
         log(f"[bench] cpu_baseline {out['cpu_baseline']}")
+    if not args.no_weave:
+        out["weave"] = weave_block(device, 40)
+        log(f"[bench] weave {out['weave']}")
     if args.calibration_copy:
         calibration_copies(device)
     if args.sweep:
@@ -678,9 +722,6 @@ def main():
                                           "gbps": round(b / r["event_us_per_launch"] / 1e3, 1),
                                           "pct_hbm_peak": round(b / r["event_us_per_launch"] / 1e3 / HBM_PEAK_GBPS * 100, 2)}
                 log(f"[sweep] {name}+{epi}: {sweep[f'{name}+{epi}']}")
-        w = time_weave(device, norm_cap=0, gemm_cap=128)
-        sweep["c5_weave"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}
-        log(f"[sweep] c5_weave: {sweep['c5_weave']}")
         out["sweep"] = sweep
     print(json.dumps(out), flush=True)
 

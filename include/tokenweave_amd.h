@@ -205,6 +205,25 @@ TW_API int tw_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M,
                     int64_t N, int64_t K, int64_t ldc, int max_cus,
                     void* stream);
 
+/* The producer of the fused op's input: the P row-parallel partial sums of one
+ * token split in ONE launch, outs[p][M, N] = as[p][M, K] * bs[p][N, K]^T for
+ * p < num_partials, each written straight into its rank's staging rows (outs[p] =
+ * slot p of the staging buffer at the split's first row, ldc = the slot's row
+ * stride in elements) — the layout tw_reduce_add_rms_norm / tw_fused_rs_ln_ag_cta
+ * read, with no copy in between.  outs, as, bs are HOST arrays of num_partials
+ * device pointers; shapes, alignment and max_cus as for tw_gemm_bf16_nt; results are
+ * bit-identical to num_partials calls of tw_gemm_bf16_nt.  Workgroups walk
+ * num_partials x tiles; with eight partials every XCD computes one of them.
+ * Replaces the row-parallel o_proj / down_proj writing in place into the symmetric
+ * staging buffer: UnquantizedLinearMethod.apply_inplace and
+ * RowParallelLinear.forward_inplace (vllm/model_executor/layers/linear.py:203-228,
+ * 1310-1321), called from vllm/model_executor/models/llama.py:99-103,248-249 —
+ * there one GEMM per rank, here (one GPU standing in for the ranks) all of them. */
+TW_API int tw_gemm_bf16_nt_partials(void* const* outs, const void* const* as,
+                             const void* const* bs, int num_partials, int64_t M,
+                             int64_t N, int64_t K, int64_t ldc, int max_cus,
+                             void* stream);
+
 /* Norm with static-scale fp8 output.  out is [num_tokens, hidden_size] of OCP
  * float8 e4m3fn (1 byte per element): out = fp8_rne(clamp(y / *scale, +-448)),
  * where y is the bf16 (or `dtype`) result the unquantised op would store, and

@@ -94,6 +94,115 @@ def test_gemm_large_tile_kernel_store_paths(M, N, K, ldc, shift):
     assert not flat[:shift].any() and not flat[shift + M * ldc:].any()
 
 
+@pytest.mark.parametrize("P,M,N,K,first_row,rows", [
+    (8, 300, 512, 128, 0, 300),       # small: every tile kind of the big kernel's edges
+    (8, 333, 8192, 1024, 200, 600),   # ragged M, the split starts at a non-zero staging row
+    (3, 645, 520, 192, 7, 700),       # odd P, ragged tiles in both directions
+    (2, 100, 128, 64, 5, 128),        # too small for the big kernel: one launch per product
+])
+def test_partials_producer_writes_every_rank_slot(P, M, N, K, first_row, rows):
+    """tw_gemm_bf16_nt_partials: the P partial sums of a token split land in rows
+    [first_row, first_row + M) of the P staging slots — each against fp32 CPU arithmetic,
+    bit-identical to P separate tw_gemm_bf16_nt calls, nothing else touched."""
+    print(f"[case] partials P={P} M={M} N={N} K={K} first_row={first_row}", flush=True)
+    gs = wl.make_partials_gemm_inputs(P, M, N, K, DEV, seed=P * 1000 + M)
+    buf = tw.PartialsBuffer(P, rows, N, rank=0, device=DEV)
+    buf.storage.fill_(float("nan"))
+    outs = [buf.slot(p)[first_row:first_row + M] for p in range(P)]
+    ops.gemm_bf16_nt_partials(outs, [g.a for g in gs], [g.b for g in gs])
+    one = tw.PartialsBuffer(P, rows, N, rank=0, device=DEV)
+    one.storage.fill_(float("nan"))
+    for p in range(P):
+        ops.gemm_bf16_nt(one.slot(p)[first_row:first_row + M], gs[p].a, gs[p].b)
+    torch.cuda.synchronize()
+    for p in range(P):
+        check(outs[p], gs[p].a, gs[p].b, f"slot {p}")
+    assert torch.equal(buf.storage.view(torch.int16), one.storage.view(torch.int16))
+    assert torch.isnan(buf.storage[:, :first_row]).all() and torch.isnan(buf.storage[:, first_row + M:]).all()
+
+
+def test_partials_producer_feeds_the_fused_norm(oracle):
+    """Producer and consumer through one staging buffer: the GEMMs' partial sums are what
+    the fused op reads, with no copy in between; checked against the CPU checker fed with
+    the GEMM outputs."""
+    P, M, N, K = 8, 96, 8192, 256
+    gs = wl.make_partials_gemm_inputs(P, M, N, K, DEV, seed=77, weight_std=0.05)
+    buf = tw.PartialsBuffer(P, M, N, rank=1, device=DEV)
+    ops.gemm_bf16_nt_partials([buf.slot(p) for p in range(P)], [g.a for g in gs], [g.b for g in gs])
+    torch.cuda.synchronize()
+    parts = [to_bits(buf.slot(p)) for p in range(P)]
+    residual = torch.randn(M, N, device=DEV).to(torch.bfloat16)
+    r0 = to_bits(residual)
+    layer = tw.RMSNorm(N, eps=1e-5, dtype=torch.bfloat16).to(DEV)
+    y, r = layer(buf.hidden_states(M), residual, MAX_CTAS=0, fused_ar=True, symm_mem_hdl=buf, rank=1,
+                 world_size=P, offset=0)
+    torch.cuda.synchronize()
+    y_want, r_want = oracle.reduce_add_rms_norm(parts, r0, to_bits(layer.weight.data), 1e-5)
+    assert np.array_equal(to_bits(r), r_want)
+    from helpers import ulp_distance
+    assert ulp_distance(to_bits(y), y_want).max() <= 1
+
+
+def test_partials_producer_argument_checks():
+    gs = wl.make_partials_gemm_inputs(2, 64, 128, 64, DEV, seed=3)
+    out = [torch.empty((64, 128), dtype=torch.bfloat16, device=DEV) for _ in range(2)]
+    with pytest.raises(RuntimeError, match="one entry per partial"):
+        ops.gemm_bf16_nt_partials(out, [gs[0].a], [g.b for g in gs])
+    with pytest.raises(RuntimeError, match="partial 1 has"):
+        ops.gemm_bf16_nt_partials([out[0], out[1][:32]], [gs[0].a, gs[1].a[:32]], [g.b for g in gs])
+    with pytest.raises(RuntimeError, match="not in"):
+        ops.gemm_bf16_nt_partials([], [], [])
+
+
+def test_config5_stage_at_full_size_equals_serial_execution():
+    """The weave configuration as it is benchmarked: the producer GEMM of the 2458-row
+    split (all eight partials, and the single-partial form) on the current stream while
+    the fused norm of the 1638-row split runs on a second stream — same bits as running
+    them in turn, and the GEMM against fp32 CPU arithmetic."""
+    P, H, K = 8, 8192, wl.C5_GEMM_K
+    T, Ta = wl.C5_TOTAL_TOKENS, wl.C5_GEMM_ROWS
+    cfg = wl.C5_NORM
+    inp = wl.make_norm_inputs(cfg, DEV)
+    gs = wl.make_partials_gemm_inputs(P, Ta, H, K, DEV)
+    layer = tw.RMSNorm(H, eps=cfg.eps, dtype=torch.bfloat16).to(DEV)
+    layer.weight.data.copy_(inp.weight)
+    rank = 3
+
+    def setup():
+        buf = tw.PartialsBuffer(P, T, H, rank=rank, device=DEV)
+        buf.storage.zero_()
+        buf.storage[:, Ta:] = inp.staging
+        residual = torch.zeros(T, H, dtype=torch.bfloat16, device=DEV)
+        residual[Ta:] = inp.residual
+        return buf, residual
+
+    def norm(buf, residual):
+        layer(buf.local[Ta:], residual[Ta:], MAX_CTAS=0, fused_ar=True, symm_mem_hdl=buf, rank=rank,
+              world_size=P, offset=buf.offset_of_row(Ta))
+
+    def gemm8(buf, cus=None):
+        ops.gemm_bf16_nt_partials([buf.slot(p)[:Ta] for p in range(P)], [g.a for g in gs], [g.b for g in gs], cus)
+
+    def gemm1(buf, cus=None):
+        ops.gemm_bf16_nt(buf.local[:Ta], gs[rank].a, gs[rank].b, cus)
+
+    side = torch.cuda.Stream()
+    for name, gemm in (("eight partials", gemm8), ("one partial", gemm1)):
+        print(f"[case] config 5 stage, {name}", flush=True)
+        buf1, res1 = setup()
+        gemm(buf1)
+        norm(buf1, res1)
+        torch.cuda.synchronize()
+        buf2, res2 = setup()
+        tw.weave_norm_gemm(lambda: gemm(buf2, 128), lambda: norm(buf2, res2), side, gemm_first=True)
+        torch.cuda.synchronize()
+        assert torch.equal(buf1.storage.view(torch.int16), buf2.storage.view(torch.int16)), name
+        assert torch.equal(res1.view(torch.int16), res2.view(torch.int16)), name
+        check(buf2.local[:Ta], gs[rank].a, gs[rank].b, f"config 5 gemm ({name})")
+        if gemm is gemm8:
+            check(buf2.slot(0)[:Ta], gs[0].a, gs[0].b, "config 5 gemm, slot 0")
+
+
 def test_weave_step_equals_serial_execution():
     """GEMM of split A on the current stream while split B's fused norm runs on a
     second stream (tokenweave_utils.py:236-260): same bits as running them in turn."""

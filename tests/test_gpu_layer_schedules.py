@@ -30,6 +30,7 @@ class ToyLayer:
         self.coef = {k: (torch.randn(WS, generator=g, device=DEV) * 0.5,
                          torch.randn(WS, H, generator=g, device=DEV) * 0.1) for k in ("attn", "mlp")}
         self.calls = []
+        self.budgets = []   # the compute-unit budget each projection was given
 
     def _project(self, kind, hidden_states):
         row_bytes = H * 2
@@ -41,13 +42,15 @@ class ToyLayer:
             self.buf.slot(p)[first:first + n].copy_((x * a[p] + b[p]).to(torch.bfloat16))
         self.calls.append((kind, int(first), int(n)))
 
-    def self_attn(self, positions, hidden_states, **kwargs):
+    def self_attn(self, positions, hidden_states, gemm_cus=None, **kwargs):
         assert positions.shape[0] == hidden_states.shape[0]
         self._project("attn", hidden_states)
+        self.budgets.append(gemm_cus)
         return hidden_states
 
-    def mlp(self, hidden_states):
+    def mlp(self, hidden_states, gemm_cus=None):
         self._project("mlp", hidden_states)
+        self.budgets.append(gemm_cus)
         return hidden_states
 
 
@@ -71,7 +74,7 @@ def torch_stack(emb, layers, final_norm):
     return x, res
 
 
-def run_stack(T, schedule):
+def run_stack(T, schedule, gemm_cus=0):
     torch.manual_seed(7)
     buf = tw.PartialsBuffer(WS, T, H, rank=RANK, device=DEV)
     layers = [ToyLayer(buf, 100 + i) for i in range(LAYERS)]
@@ -96,7 +99,7 @@ def run_stack(T, schedule):
                 layer, positions, hidden_states, residual, buf, i, end_layer=LAYERS, rank=RANK,
                 world_size=WS, current_stream=cur, copy_stream=side, next_layer_norm=nxt,
                 split_size=split, actual_tokens=T, num_tokens_padded=T, MAX_CTAS_ATTN=16,
-                MAX_CTAS_MLP=16, mlp_fn=layer.mlp, all_ranks=True)
+                MAX_CTAS_MLP=16, mlp_fn=layer.mlp, all_ranks=True, gemm_cus=gemm_cus)
     torch.cuda.synchronize()
     return hidden_states.clone(), residual.clone(), emb, layers, final_norm, split
 
@@ -111,6 +114,20 @@ def test_overlap_schedule_equals_fuse_only_schedule(T):
     y_ref, r_ref = torch_stack(emb, layers, final_norm)
     torch.testing.assert_close(r0.float(), r_ref.float(), rtol=RTOL, atol=ATOL)
     torch.testing.assert_close(y0.float(), y_ref.float(), rtol=RTOL, atol=ATOL)
+
+
+def test_overlap_schedule_hands_the_gemm_budget_of_the_plan_to_the_projections():
+    """weave_plan's gemm_cus reaches every projection that runs beside a norm; without a
+    budget the layer's callables are called with the reference's keywords only."""
+    T = 4096
+    plan = tw.weave_plan(T, tw.load_config("tokenweave_configs/llama_config_8.json"))
+    assert plan is not None and plan["gemm_cus"] > 0
+    y0, r0, _, layers, _, _ = run_stack(1000, "overlap", gemm_cus=plan["gemm_cus"])
+    for layer in layers:
+        assert layer.budgets == [plan["gemm_cus"]] * 4
+    y1, r1, _, layers, _, _ = run_stack(1000, "overlap")
+    assert all(layer.budgets == [None] * 4 for layer in layers)
+    assert torch.equal(y0, y1) and torch.equal(r0, r1)
 
 
 def test_fuse_only_touches_only_this_ranks_shard_without_all_ranks():

@@ -625,6 +625,41 @@ def bind_gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
     return BoundOp(*_prepare_gemm_bf16_nt(out, a, b, max_cus))
 
 
+def _prepare_gemm_bf16_nt_partials(outs, a_list, b_list, max_cus):
+    P = len(outs)
+    _require(1 <= P <= _lib.TW_MAX_PARTIALS, f"number of partials {P} not in [1, {_lib.TW_MAX_PARTIALS}]")
+    _require(len(a_list) == P and len(b_list) == P, "outs, a and b must have one entry per partial")
+    shape = None
+    for p in range(P):
+        # the per-product checks of gemm_bf16_nt; all products must share one shape and row stride
+        _, args, _, dev = _prepare_gemm_bf16_nt(outs[p], a_list[p], b_list[p], max_cus)
+        if shape is None:
+            shape, dev0 = args[3:7], dev
+        _require(args[3:7] == shape and dev == dev0,
+                 f"partial {p} has (M, N, K, row stride) {args[3:7]}, partial 0 has {shape}")
+    vp = ctypes.c_void_p
+    o = (vp * P)(*[t.data_ptr() for t in outs])
+    a = (vp * P)(*[t.data_ptr() for t in a_list])
+    b = (vp * P)(*[t.data_ptr() for t in b_list])
+    args = (o, a, b, P, *shape, _cap(max_cus))
+    return _lib.lib().tw_gemm_bf16_nt_partials, args, (list(outs), list(a_list), list(b_list)), dev0
+
+
+def gemm_bf16_nt_partials(outs: Sequence[torch.Tensor], a: Sequence[torch.Tensor], b: Sequence[torch.Tensor],
+                          max_cus: Optional[int] = None) -> None:
+    """outs[p][M, N] <- a[p][M, K] @ b[p][N, K]^T for every p in ONE launch: the P row-parallel
+    partial sums of a token split, each written straight into its rank's staging rows
+    (`outs[p]` = `PartialsBuffer.slot(p)[first_row:first_row + M]`).  The producer side of
+    the fused op: vllm/model_executor/layers/linear.py:203-228, 1310-1321."""
+    BoundOp(*_prepare_gemm_bf16_nt_partials(outs, a, b, max_cus))()
+
+
+def bind_gemm_bf16_nt_partials(outs: Sequence[torch.Tensor], a: Sequence[torch.Tensor],
+                               b: Sequence[torch.Tensor], max_cus: Optional[int] = None) -> BoundOp:
+    """`gemm_bf16_nt_partials` with the checks done now and the launch deferred."""
+    return BoundOp(*_prepare_gemm_bf16_nt_partials(outs, a, b, max_cus))
+
+
 def num_compute_units(device=None) -> int:
     dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
     with torch.cuda.device(dev):

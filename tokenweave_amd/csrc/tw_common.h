@@ -70,6 +70,9 @@ int split_segments(int64_t T, int64_t H, int max_ctas);
 int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t N,
                      int64_t K, int64_t ldc, int max_cus, void* stream);
 
+int run_gemm_bf16_nt_partials(void* const* outs, const void* const* as, const void* const* bs, int count,
+                              int64_t M, int64_t N, int64_t K, int64_t ldc, int max_cus, void* stream);
+
 }  // namespace tw
 
 #endif

@@ -205,10 +205,18 @@ __device__ __forceinline__ void big_issue_slab(__amdgpu_buffer_rsrc_t da, __amdg
     __builtin_amdgcn_raw_ptr_buffer_load_lds(db, (lds_void_t*)(sb + j * 1024), 16, vb[j], koff, 0, 0);
 }
 
+// `count` independent products of one shape in one launch: out[p] = a[p] * b[p]^T.  The
+// token-weave producer uses it for the P row-parallel partial sums of a token split,
+// each written into its rank's staging slot; a plain GEMM is count = 1.
+struct GemmBatch {
+  uint16_t* out[TW_MAX_PARTIALS];
+  const uint16_t* a[TW_MAX_PARTIALS];
+  const uint16_t* b[TW_MAX_PARTIALS];
+};
+
 template <int TM, int TN>
 __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
-    uint16_t* __restrict__ out, const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
-    int M, int N, int K, int64_t ldc, int tiles_m, int tiles_n, int wide_store) {
+    GemmBatch batch, int count, int M, int N, int K, int64_t ldc, int tiles_m, int tiles_n, int wide_store) {
   constexpr int WM = 32 * TM, WN = 32 * TN;  // wave tile
   constexpr int BM = 2 * WM, BN = 4 * WN;    // workgroup tile: the 8 waves as 2 x 4
   constexpr int PANEL_A = BM * BIG_ROWB;
@@ -220,7 +228,8 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 2, wn = wave & 3, l32 = lane & 31, lhi = lane >> 5;
-  const int num_tiles = tiles_m * tiles_n;
+  const int tiles_per_product = tiles_m * tiles_n;
+  const int num_tiles = count * tiles_per_product;
   const int nk = K / BIG_BK;
   // Loader: wave instruction j of wave w fills the 8-row LDS block w * L + j; lane l
   // lands at row l / 8, position l % 8 of that block, so it must fetch the chunk
@@ -234,18 +243,22 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
   for (int kk = 0; kk < 4; ++kk)
     roff[kk] = l32 * BIG_ROWB + ((((kk << 1) | lhi) ^ ((l32 >> 1) & 7)) << 4);
 
-  const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(a), 0, (uint32_t)((size_t)M * K * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(b), 0, (uint32_t)((size_t)N * K * 2), 0x00020000);
-
   for (int t = blockIdx.x; t < num_tiles; t += gridDim.x) {
+    // Every XCD (workgroup ids congruent mod 8) gets a contiguous range of the tile order:
+    // with eight products, one product each.
     int pid = t;
     {
       const int per_xcd = num_tiles / 8;
       const int body = per_xcd * 8;
       if (t < body) pid = (t & 7) * per_xcd + (t >> 3);
     }
+    const int product = pid / tiles_per_product;
+    pid -= product * tiles_per_product;
+    uint16_t* __restrict__ out = batch.out[product];
+    const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(batch.a[product]), 0, (uint32_t)((size_t)M * K * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(batch.b[product]), 0, (uint32_t)((size_t)N * K * 2), 0x00020000);
     const int group_size = BIG_GROUP_M * tiles_n;
     const int group = pid / group_size;
     const int first_m = group * BIG_GROUP_M;
@@ -449,8 +462,8 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
 }
 
 template <int TM, int TN>
-static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64_t M, int64_t N,
-                      int64_t K, int64_t ldc, int max_cus, hipStream_t hs) {
+static int launch_big(const GemmBatch& batch, int count, int64_t M, int64_t N, int64_t K, int64_t ldc,
+                      int max_cus, hipStream_t hs) {
   constexpr int BM = 64 * TM, BN = 128 * TN;
   constexpr int LDS = big_lds_bytes(TM, TN);
   // the attribute belongs to the function on one device: set it once per device
@@ -466,11 +479,13 @@ static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64
     lds_ok[dev].store(true, std::memory_order_release);
   }
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
-  int64_t grid = (int64_t)tiles_m * tiles_n;
+  int64_t grid = (int64_t)count * tiles_m * tiles_n;
   if (max_cus > 0 && grid > max_cus) grid = max_cus;
   // 16-byte stores need 16-byte aligned row segments that end inside the row
-  const int wide_store = (N % 8 == 0 && ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) ? 1 : 0;
-  launch_kernel(gemm_bf16_nt_big_kernel<TM, TN>, dim3((unsigned)grid), dim3(BIG_THREADS), LDS, hs, out, a, b,
+  int wide_store = (N % 8 == 0 && ldc % 8 == 0) ? 1 : 0;
+  for (int p = 0; p < count; ++p)
+    if (reinterpret_cast<uintptr_t>(batch.out[p]) & 15u) wide_store = 0;
+  launch_kernel(gemm_bf16_nt_big_kernel<TM, TN>, dim3((unsigned)grid), dim3(BIG_THREADS), LDS, hs, batch, count,
                 (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n, wide_store);
   return TW_OK;
 }
@@ -485,7 +500,7 @@ static int launch_big(uint16_t* out, const uint16_t* a, const uint16_t* b, int64
 // 256 x 256 and are not offered.
 struct BigTile { int tm, tn; };
 
-static BigTile pick_big_tile(int64_t M, int64_t N, int cus) {
+static BigTile pick_big_tile(int64_t M, int64_t N, int count, int cus) {
   // Relative throughput per tile area, measured: the 256 x 384 tile loads a fifth fewer
   // operand bytes per flop and runs a round in 1.35x the time of a 256 x 256 round.
   static const struct { int tm, tn; double eff; } kTiles[] = {
@@ -493,7 +508,7 @@ static BigTile pick_big_tile(int64_t M, int64_t N, int cus) {
   BigTile best = {4, 2};
   double best_cost = 1e300;
   for (const auto& t : kTiles) {
-    const int64_t tiles = ((M + 64 * t.tm - 1) / (64 * t.tm)) * ((N + 128 * t.tn - 1) / (128 * t.tn));
+    const int64_t tiles = count * ((M + 64 * t.tm - 1) / (64 * t.tm)) * ((N + 128 * t.tn - 1) / (128 * t.tn));
     const int64_t rounds = (tiles + cus - 1) / cus;
     const double cost = (double)rounds * (64.0 * t.tm * 128.0 * t.tn / t.eff + 2048.0);
     if (cost < best_cost) {
@@ -504,37 +519,56 @@ static BigTile pick_big_tile(int64_t M, int64_t N, int cus) {
   return best;
 }
 
+// The tile shape never changes a result bit: every output element is the same sequence of
+// MFMA k-steps whatever tile it lies in.
+static bool big_kernel_fits(int64_t M, int64_t N, int64_t K) {
+  // whole 64-wide k-slabs, 32-bit byte offsets into both operands, and enough rows and
+  // columns to be worth the larger prologue
+  return (K % BIG_BK == 0) && ((uint64_t)M * K < (1ull << 31)) && ((uint64_t)N * K < (1ull << 31)) && M >= 192 &&
+         N >= 192;
+}
+
+static int launch_big_for(const GemmBatch& batch, int count, int64_t M, int64_t N, int64_t K, int64_t ldc,
+                          int max_cus, hipStream_t hs) {
+  int cus = max_cus > 0 ? max_cus : device_compute_units();
+  if (cus <= 0) cus = 256;
+  const BigTile bt = pick_big_tile(M, N, count, cus);
+  if (bt.tn == 3) return launch_big<4, 3>(batch, count, M, N, K, ldc, max_cus, hs);
+  if (bt.tm == 2) return launch_big<2, 2>(batch, count, M, N, K, ldc, max_cus, hs);
+  if (bt.tm == 3) return launch_big<3, 2>(batch, count, M, N, K, ldc, max_cus, hs);
+  if (bt.tm == 5) return launch_big<5, 2>(batch, count, M, N, K, ldc, max_cus, hs);
+  return launch_big<4, 2>(batch, count, M, N, K, ldc, max_cus, hs);
+}
+
+static int check_gemm_shape(const char* what, int64_t M, int64_t N, int64_t K, int64_t ldc) {
+  if (M < 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || ldc < N)
+    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: bad shape M=%lld N=%lld K=%lld ldc=%lld", what, (long long)M,
+                     (long long)N, (long long)K, (long long)ldc);
+  if (K % 8 != 0 || N % 4 != 0 || ldc % 4 != 0)
+    return set_error(TW_ERR_ALIGNMENT, "%s: needs K %% 8 == 0, N %% 4 == 0, ldc %% 4 == 0", what);
+  return TW_OK;
+}
+
+static int check_gemm_pointers(const char* what, const void* out, const void* a, const void* b) {
+  if (!out || !a || !b) return set_error(TW_ERR_INVALID_ARGUMENT, "%s: null pointer argument", what);
+  auto al = [](const void* p, unsigned n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) == 0; };
+  if (!al(a, 16) || !al(b, 16) || !al(out, 8))
+    return set_error(TW_ERR_ALIGNMENT, "%s: needs 16-byte aligned a and b, 8-byte aligned out", what);
+  return TW_OK;
+}
+
 int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t N, int64_t K,
                      int64_t ldc, int max_cus, void* stream) {
-  if (M < 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || ldc < N)
-    return set_error(TW_ERR_INVALID_ARGUMENT, "gemm_bf16_nt: bad shape M=%lld N=%lld K=%lld ldc=%lld",
-                     (long long)M, (long long)N, (long long)K, (long long)ldc);
+  if (int rc = check_gemm_shape("gemm_bf16_nt", M, N, K, ldc)) return rc;
   if (M == 0) return TW_OK;
-  if (!out || !a || !b) return set_error(TW_ERR_INVALID_ARGUMENT, "gemm_bf16_nt: null pointer argument");
-  auto al = [](const void* p, unsigned n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) == 0; };
-  if (K % 8 != 0 || N % 4 != 0 || ldc % 4 != 0 || !al(a, 16) || !al(b, 16) || !al(out, 8))
-    return set_error(TW_ERR_ALIGNMENT,
-                     "gemm_bf16_nt: needs K %% 8 == 0, N %% 4 == 0, ldc %% 4 == 0, 16-byte aligned "
-                     "a and b, 8-byte aligned out");
+  if (int rc = check_gemm_pointers("gemm_bf16_nt", out, a, b)) return rc;
   hipStream_t hs = static_cast<hipStream_t>(stream);
-  // The 256 x 256 kernel needs whole 64-wide k-slabs, 32-bit byte offsets into both
-  // operands and enough tiles to be worth its larger prologue.
-  const bool big = (K % BIG_BK == 0) && ((uint64_t)M * K < (1ull << 31)) && ((uint64_t)N * K < (1ull << 31)) &&
-                   M >= 192 && N >= 192;
-  if (big) {
-    int cus = max_cus > 0 ? max_cus : device_compute_units();
-    if (cus <= 0) cus = 256;
-    uint16_t* o = static_cast<uint16_t*>(out);
-    const uint16_t* pa = static_cast<const uint16_t*>(a);
-    const uint16_t* pb = static_cast<const uint16_t*>(b);
-    int rc;
-    const BigTile bt = pick_big_tile(M, N, cus);
-    if (bt.tn == 3) rc = launch_big<4, 3>(o, pa, pb, M, N, K, ldc, max_cus, hs);
-    else if (bt.tm == 2) rc = launch_big<2, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
-    else if (bt.tm == 3) rc = launch_big<3, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
-    else if (bt.tm == 5) rc = launch_big<5, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
-    else rc = launch_big<4, 2>(o, pa, pb, M, N, K, ldc, max_cus, hs);
-    if (rc != TW_OK) return rc;
+  if (big_kernel_fits(M, N, K)) {
+    GemmBatch batch = {};
+    batch.out[0] = static_cast<uint16_t*>(out);
+    batch.a[0] = static_cast<const uint16_t*>(a);
+    batch.b[0] = static_cast<const uint16_t*>(b);
+    if (int rc = launch_big_for(batch, 1, M, N, K, ldc, max_cus, hs)) return rc;
   } else {
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
     int64_t grid = (int64_t)tiles_m * tiles_n;
@@ -545,6 +579,33 @@ int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t
                   static_cast<const uint16_t*>(b), (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n);
   }
   return finish_launch("gemm_bf16_nt");
+}
+
+// outs[p][M, N] (row stride ldc) = as[p][M, K] * bs[p][N, K]^T for p < count: one launch
+// over count x tiles when the shape fits the big kernel, one launch per product otherwise.
+int run_gemm_bf16_nt_partials(void* const* outs, const void* const* as, const void* const* bs, int count,
+                              int64_t M, int64_t N, int64_t K, int64_t ldc, int max_cus, void* stream) {
+  const char* what = "gemm_bf16_nt_partials";
+  if (count < 1 || count > TW_MAX_PARTIALS)
+    return set_error(TW_ERR_INVALID_ARGUMENT, "%s: number of partials %d not in [1, %d]", what, count,
+                     TW_MAX_PARTIALS);
+  if (int rc = check_gemm_shape(what, M, N, K, ldc)) return rc;
+  if (M == 0) return TW_OK;
+  if (!outs || !as || !bs) return set_error(TW_ERR_INVALID_ARGUMENT, "%s: null pointer argument", what);
+  GemmBatch batch = {};
+  for (int p = 0; p < count; ++p) {
+    if (int rc = check_gemm_pointers(what, outs[p], as[p], bs[p])) return rc;
+    batch.out[p] = static_cast<uint16_t*>(outs[p]);
+    batch.a[p] = static_cast<const uint16_t*>(as[p]);
+    batch.b[p] = static_cast<const uint16_t*>(bs[p]);
+  }
+  if (big_kernel_fits(M, N, K)) {
+    if (int rc = launch_big_for(batch, count, M, N, K, ldc, max_cus, static_cast<hipStream_t>(stream))) return rc;
+    return finish_launch(what);
+  }
+  for (int p = 0; p < count; ++p)
+    if (int rc = run_gemm_bf16_nt(outs[p], as[p], bs[p], M, N, K, ldc, max_cus, stream)) return rc;
+  return TW_OK;
 }
 
 }  // namespace tw

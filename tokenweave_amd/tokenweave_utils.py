@@ -306,6 +306,7 @@ def tokenweave_overlap(
     MAX_CTAS_MLP: int = 16,
     mlp_fn: Optional[Callable] = None,
     all_ranks: bool = False,
+    gemm_cus: int = 0,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """One decoder layer under the TokenWeave schedule (reference
     tokenweave_utils.py:175-340, same arguments and the same order of hand-offs):
@@ -320,6 +321,13 @@ def tokenweave_overlap(
     normalises its shard and all-gathers — on one GPU that is the fused op on a
     zeroed residual (residual <- sum of the partials, x <- norm of it).
     The last layer normalises split 1 after its MLP on the current stream (:327-339).
+
+    `gemm_cus` (no counterpart in the reference; `weave_plan(...)["gemm_cus"]`) is the
+    compute-unit budget of the GEMMs that run beside a norm: when non-zero it is handed to
+    `self.self_attn(..., gemm_cus=)` and `mlp_fn(hidden_states, gemm_cus=)`, which pass it as
+    `max_cus` to their row-parallel output projection (`ops.gemm_bf16_nt` /
+    `ops.gemm_bf16_nt_partials`) so that the norm's workgroups find free compute units.  On
+    MI355X that, not the norm's grid cap, is the knob of the overlap.
 
     The two norms that the reference launches with hard-coded grids (8 CTAs in layer
     0, 16 or 32 after the last layer) have nothing to share the GPU with and are
@@ -336,6 +344,8 @@ def tokenweave_overlap(
     blpr_2 = hidden_states_2.shape[0] // world_size
     rows_1 = _shard_rows(split_size, rank, world_size, all_ranks)
     rows_2 = _shard_rows(hidden_states_2.shape[0], rank, world_size, all_ranks)
+
+    budget = {"gemm_cus": gemm_cus} if gemm_cus else {}
 
     def norm(layernorm, split, max_ctas):
         hs, res, blpr, off, rows = ((hidden_states_1, residual_1, blpr_1, 0, rows_1) if split == 0 else
@@ -356,7 +366,7 @@ def tokenweave_overlap(
 
     with torch.cuda.stream(current_stream):
         self.self_attn(positions=positions[:split_size], hidden_states=hidden_states_1, split_id=0,
-                       split_size=split_size, num_actual_tokens=split_size)
+                       split_size=split_size, num_actual_tokens=split_size, **budget)
         current_stream.wait_stream(copy_stream)
     with torch.cuda.stream(copy_stream):
         copy_stream.wait_stream(current_stream)
@@ -364,21 +374,21 @@ def tokenweave_overlap(
 
     with torch.cuda.stream(current_stream):
         self.self_attn(positions=positions[split_size:], hidden_states=hidden_states_2, split_id=1,
-                       split_size=split_size, num_actual_tokens=actual_tokens - split_size)
+                       split_size=split_size, num_actual_tokens=actual_tokens - split_size, **budget)
         current_stream.wait_stream(copy_stream)
     with torch.cuda.stream(copy_stream):
         copy_stream.wait_stream(current_stream)
         norm(self.post_attention_layernorm, 1, MAX_CTAS_MLP)
 
     with torch.cuda.stream(current_stream):
-        mlp_fn(hidden_states_1)
+        mlp_fn(hidden_states_1, **budget)
         current_stream.wait_stream(copy_stream)
     with torch.cuda.stream(copy_stream):
         copy_stream.wait_stream(current_stream)
         norm(next_layer_norm, 0, MAX_CTAS_MLP)
 
     with torch.cuda.stream(current_stream):
-        mlp_fn(hidden_states_2)
+        mlp_fn(hidden_states_2, **budget)
         current_stream.wait_stream(copy_stream)
 
     if layer_id == end_layer - 1:

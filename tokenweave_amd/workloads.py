@@ -126,6 +126,14 @@ class GemmInputs:
     b: torch.Tensor   # [N, K] bf16 weight (row-parallel slice of o_proj)
 
 
+def make_partials_gemm_inputs(P: int = 8, M: int = C5_GEMM_ROWS, N: int = 8192, K: int = C5_GEMM_K,
+                              device="cuda", seed: int = C5_NORM.seed + 2,
+                              weight_std: float = C5_WEIGHT_STD) -> List["GemmInputs"]:
+    """The row-parallel GEMMs of P simulated ranks on one token split: rank p holds its own
+    K-slice of the activations and of the weight."""
+    return [make_gemm_inputs(M, N, K, device, seed + 101 * p, weight_std) for p in range(P)]
+
+
 def make_gemm_inputs(M: int = C5_GEMM_ROWS, N: int = 8192, K: int = C5_GEMM_K, device="cuda",
                      seed: int = C5_NORM.seed + 1, weight_std: float = C5_WEIGHT_STD) -> GemmInputs:
     dev = torch.device(device)

@@ -102,6 +102,8 @@ def parse_args():
     ap.add_argument("--ceilings", action="store_true",
                     help="time the memory-system yardsticks (read-only row streams, the norm's traffic "
                          "without arithmetic, plain copy, empty kernel) at 256 and 2048 rows and print them")
+    ap.add_argument("--host-cost", action="store_true",
+                    help="measure the host time per call of the op's entry routes and print it")
     ap.add_argument("--timeline", action="store_true",
                     help="run the workload through the stamped build of the norm kernel and print the "
                          "per-workgroup timeline breakdown")
@@ -447,6 +449,58 @@ def time_arrivals(cfg, device, launches=100):
     return out
 
 
+def host_cost(device, calls=3000):
+    """Host time per call (the loop's wall time without a device synchronisation; the GPU
+    queue is deep enough not to block it) of the ways into the op, on a decode-size batch
+    (8 rows, P = 8, H = 8192), with torch.add as the yardstick.  Microseconds."""
+    import torch
+    import tokenweave_amd as tw
+    from tokenweave_amd import _custom_ops as ops
+    T, H, P = 8, 8192, 8
+    buf = tw.PartialsBuffer(P, T, H, rank=0, device=device)
+    buf.storage.normal_()
+    res = torch.randn(T, H, device=device).bfloat16()
+    layer = tw.RMSNorm(H, eps=1e-5, dtype=torch.bfloat16).to(device)
+    hs = buf.hidden_states(T)
+    parts = [buf.slot(p)[:T] for p in range(P)]
+    w = layer.weight.data
+    x = torch.randn(T, H, device=device).bfloat16()
+    bound = ops.bind_reduce_add_rms_norm(parts, parts[0], res, w, 1e-5)
+    st = torch.cuda.current_stream()
+    mc = buf.multicast_ptr
+    ways = {
+        "BoundOp(stream)": lambda: bound(st),
+        "ops.fused_add_rms_norm": lambda: ops.fused_add_rms_norm(hs, res, w, 1e-5),
+        "torch.ops.tokenweave_amd.fused_add_rms_norm": lambda: torch.ops.tokenweave_amd.fused_add_rms_norm(hs, res, w, 1e-5),
+        "ops.via_ctypes.fused_add_rms_norm": lambda: ops.via_ctypes.fused_add_rms_norm(hs, res, w, 1e-5),
+        "ops.fused_rs_ln_ag_cta": lambda: ops.fused_rs_ln_ag_cta(hs, res, w, mc, 0, 0, P, 0, 1e-5),
+        "ops.via_ctypes.fused_rs_ln_ag_cta": lambda: ops.via_ctypes.fused_rs_ln_ag_cta(hs, res, w, mc, 0, 0, P, 0, 1e-5),
+        "ops.reduce_add_rms_norm(8 tensors)": lambda: ops.reduce_add_rms_norm(parts, parts[0], res, w, 1e-5),
+        "RMSNorm(x, residual)": lambda: layer(hs, res),
+        "RMSNorm(x, residual, fused_ar=True, ...)": lambda: layer(hs, res, MAX_CTAS=None, fused_ar=True,
+                                                                   symm_mem_hdl=buf, rank=0, world_size=P, offset=0),
+        "fused_allreduce_layernorm": lambda: tw.fused_allreduce_layernorm(layer, hs, res, buf, T // P, 0, P, 0),
+        "torch.add(x, x, out=x)": lambda: torch.add(x, x, out=x),
+    }
+    out = {"compiled_binding": bool(ops.COMPILED_BINDING), "calls": calls}
+    for name, fn in ways.items():
+        for _ in range(200):
+            fn()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for _ in range(calls):
+                fn()
+            t1 = time.perf_counter()
+            torch.cuda.synchronize()
+            us = (t1 - t0) * 1e6 / calls
+            best = us if best is None else min(best, us)
+        out[name] = round(best, 2)
+        log(f"[host] {name}: {best:.2f} us")
+    return out
+
+
 def time_norm_warm(cfg, steps, max_ctas, device):
     """Same call on ONE input set, so that after the first step the operands sit in
     the last-level cache (what a caller sees when the partials were just written)."""
@@ -626,6 +680,9 @@ def main():
     cfg = cfgs[args.workload]
     if args.ceilings:
         print(json.dumps({"ceilings": time_ceilings(device)}), flush=True)
+        return
+    if args.host_cost:
+        print(json.dumps({"host_us_per_call": host_cost(device)}), flush=True)
         return
     if args.timeline:
         print(json.dumps({"timeline": time_timeline(cfg, device), "arrivals": time_arrivals(cfg, device)}),

@@ -15,6 +15,9 @@ from __future__ import annotations
 
 import bisect
 import ctypes
+import itertools
+import os
+import types
 import threading
 import weakref
 from typing import Dict, List, Optional, Sequence, Tuple
@@ -25,6 +28,19 @@ from . import _lib
 
 _DTYPE_CODE = {torch.bfloat16: _lib.TW_DTYPE_BF16, torch.float16: _lib.TW_DTYPE_F16,
                torch.float32: _lib.TW_DTYPE_F32}
+
+# The ops registered with torch's dispatcher by the compiled binding
+# (csrc/tw_torch_binding.cpp -> libtokenweave_amd_torch.so, TORCH_LIBRARY with the
+# reference's schema strings).  When it has been built the public functions of this
+# module are one call into it, as vllm/_custom_ops.py is one call into torch.ops._C;
+# without it the same schemas are registered from Python further down and every op
+# goes through ctypes (`via_ctypes` always names that route).
+BINDING_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtokenweave_amd_torch.so")
+COMPILED_BINDING = False
+if os.path.exists(BINDING_PATH) and os.environ.get("TOKENWEAVE_AMD_NO_COMPILED_BINDING") != "1":
+    torch.ops.load_library(BINDING_PATH)
+    COMPILED_BINDING = True
+_T = torch.ops.tokenweave_amd
 
 # Message of the reference's launchers (csrc/tokenweave_fused_kernels.cu:259).
 ALIGNMENT_MESSAGE = ("Input, residual, and weight tensors must be 16-byte aligned and "
@@ -207,6 +223,7 @@ def fused_add_rms_norm_cta(input: torch.Tensor, residual: torch.Tensor, weight: 
 _REGIONS: List[Tuple[int, int, int, int, "weakref.ref"]] = []  # (base, stride, slots, usable, owner)
 _REGION_BASES: List[int] = []
 _REGIONS_LOCK = threading.Lock()
+_REGION_TOKENS = itertools.count(1)
 _LAST_REGION: Optional[Tuple[int, int, int, int, "weakref.ref"]] = None
 
 
@@ -221,6 +238,11 @@ def register_partials_region(base_ptr: int, stride_bytes: int, slots: int, owner
     usable = int(stride_bytes if usable_bytes is None else usable_bytes)
     _require(0 < usable <= stride_bytes, "usable bytes of a slot must fit its stride")
     entry = (int(base_ptr), int(stride_bytes), int(slots), usable, weakref.ref(owner))
+    if COMPILED_BINDING:
+        # the compiled ops keep their own table; the entry goes when the owner does
+        token = next(_REGION_TOKENS)
+        _T.register_partials_region(entry[0], entry[1], entry[2], usable, token)
+        weakref.finalize(owner, _T.unregister_partials_region, entry[0], token)
     with _REGIONS_LOCK:
         live = [r for r in _REGIONS if r[4]() is not None and r[0] != entry[0]]
         live.append(entry)
@@ -720,8 +742,73 @@ def _no_cpu(name):
     return impl
 
 
-_library = torch.library.Library("tokenweave_amd", "DEF")
-for _name, _schema in SCHEMAS.items():
-    _library.define(_schema)
-    _library.impl(_name, _IMPLS[_name], "CUDA")
-    _library.impl(_name, _no_cpu(_name), "CPU")
+via_ctypes = types.SimpleNamespace(
+    rms_norm=rms_norm, fused_add_rms_norm=fused_add_rms_norm, rms_norm_inplace=rms_norm_inplace,
+    fused_rs_ln_ag_cta=fused_rs_ln_ag_cta, fused_add_rms_norm_cta=fused_add_rms_norm_cta,
+    fused_rs_ln_cta=fused_rs_ln_cta, rms_norm_static_fp8_quant=rms_norm_static_fp8_quant,
+    fused_add_rms_norm_static_fp8_quant=fused_add_rms_norm_static_fp8_quant,
+    rms_norm_dynamic_per_token_quant_out=rms_norm_dynamic_per_token_quant_out)
+
+if COMPILED_BINDING:
+    # One dispatcher call per op (the overload is resolved once, here); the argument
+    # checks and the launch are the binding's.
+    _op_rms_norm = _T.rms_norm.default
+    _op_fused_add_rms_norm = _T.fused_add_rms_norm.default
+    _op_rms_norm_inplace = _T.rms_norm_inplace.default
+    _op_fused_add_rms_norm_cta = _T.fused_add_rms_norm_cta.default
+    _op_fused_rs_ln_ag_cta = _T.fused_rs_ln_ag_cta.default
+    _op_fused_rs_ln_cta = _T.fused_rs_ln_cta.default
+    _op_rms_norm_static_fp8_quant = _T.rms_norm_static_fp8_quant.default
+    _op_fused_add_rms_norm_static_fp8_quant = _T.fused_add_rms_norm_static_fp8_quant.default
+    _op_rms_norm_dynamic_per_token_quant = _T.rms_norm_dynamic_per_token_quant.default
+
+    def rms_norm(out: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,  # noqa: F811
+                 epsilon: float) -> None:
+        _op_rms_norm(out, input, weight, epsilon)
+
+    def fused_add_rms_norm(input: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,  # noqa: F811
+                           epsilon: float) -> None:
+        _op_fused_add_rms_norm(input, residual, weight, epsilon)
+
+    def rms_norm_inplace(out: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,  # noqa: F811
+                         epsilon: float) -> None:
+        _op_rms_norm_inplace(out, input, weight, epsilon)
+
+    def fused_add_rms_norm_cta(input: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,  # noqa: F811
+                               MAX_CTAS: int, epsilon: float) -> None:
+        _op_fused_add_rms_norm_cta(input, residual, weight, 0 if MAX_CTAS is None else MAX_CTAS, epsilon)
+
+    def fused_rs_ln_ag_cta(input: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,  # noqa: F811
+                           mcptr: int, signal_pads: int, rank: int, world_size: int, MAX_CTAS: int,
+                           epsilon: float) -> None:
+        _op_fused_rs_ln_ag_cta(input, residual, weight, mcptr, signal_pads, rank, world_size,
+                               0 if MAX_CTAS is None else MAX_CTAS, epsilon)
+
+    def fused_rs_ln_cta(input: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,  # noqa: F811
+                        mcptr: int, signal_pads: int, rank: int, world_size: int, MAX_CTAS: int,
+                        epsilon: float) -> None:
+        _op_fused_rs_ln_cta(input, residual, weight, mcptr, signal_pads, rank, world_size,
+                            0 if MAX_CTAS is None else MAX_CTAS, epsilon)
+
+    def rms_norm_static_fp8_quant(result: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,  # noqa: F811
+                                  scale: torch.Tensor, epsilon: float) -> None:
+        _op_rms_norm_static_fp8_quant(result, input, weight, scale, epsilon)
+
+    def fused_add_rms_norm_static_fp8_quant(result: torch.Tensor, input: torch.Tensor,  # noqa: F811
+                                            residual: torch.Tensor, weight: torch.Tensor,
+                                            scale: torch.Tensor, epsilon: float) -> None:
+        _op_fused_add_rms_norm_static_fp8_quant(result, input, residual, weight, scale, epsilon)
+
+    def rms_norm_dynamic_per_token_quant_out(result: torch.Tensor, input: torch.Tensor,  # noqa: F811
+                                             weight: torch.Tensor, scale: torch.Tensor, epsilon: float,
+                                             scale_ub: Optional[torch.Tensor] = None,
+                                             residual: Optional[torch.Tensor] = None) -> None:
+        """The registered op (schema csrc/torch_bindings.cpp:216-219): result, scale and
+        residual are written in place."""
+        _op_rms_norm_dynamic_per_token_quant(result, input, weight, scale, epsilon, scale_ub, residual)
+else:
+    _library = torch.library.Library("tokenweave_amd", "DEF")
+    for _name, _schema in SCHEMAS.items():
+        _library.define(_schema)
+        _library.impl(_name, _IMPLS[_name], "CUDA")
+        _library.impl(_name, _no_cpu(_name), "CPU")

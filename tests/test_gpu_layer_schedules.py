@@ -74,7 +74,7 @@ def torch_stack(emb, layers, final_norm):
     return x, res
 
 
-def run_stack(T, schedule, gemm_cus=0):
+def run_stack(T, schedule, gemm_cus=0, mlp_gemm_cus=None):
     torch.manual_seed(7)
     buf = tw.PartialsBuffer(WS, T, H, rank=RANK, device=DEV)
     layers = [ToyLayer(buf, 100 + i) for i in range(LAYERS)]
@@ -99,7 +99,8 @@ def run_stack(T, schedule, gemm_cus=0):
                 layer, positions, hidden_states, residual, buf, i, end_layer=LAYERS, rank=RANK,
                 world_size=WS, current_stream=cur, copy_stream=side, next_layer_norm=nxt,
                 split_size=split, actual_tokens=T, num_tokens_padded=T, MAX_CTAS_ATTN=16,
-                MAX_CTAS_MLP=16, mlp_fn=layer.mlp, all_ranks=True, gemm_cus=gemm_cus)
+                MAX_CTAS_MLP=16, mlp_fn=layer.mlp, all_ranks=True, gemm_cus=gemm_cus,
+                mlp_gemm_cus=mlp_gemm_cus)
     torch.cuda.synchronize()
     return hidden_states.clone(), residual.clone(), emb, layers, final_norm, split
 
@@ -119,12 +120,12 @@ def test_overlap_schedule_equals_fuse_only_schedule(T):
 def test_overlap_schedule_hands_the_gemm_budget_of_the_plan_to_the_projections():
     """weave_plan's gemm_cus reaches every projection that runs beside a norm; without a
     budget the layer's callables are called with the reference's keywords only."""
-    T = 4096
-    plan = tw.weave_plan(T, tw.load_config("tokenweave_configs/llama_config_8.json"))
-    assert plan is not None and plan["gemm_cus"] > 0
-    y0, r0, _, layers, _, _ = run_stack(1000, "overlap", gemm_cus=plan["gemm_cus"])
-    for layer in layers:
-        assert layer.budgets == [plan["gemm_cus"]] * 4
+    plan = tw.weave_plan(16384, tw.load_config("tokenweave_configs/llama_config_8.json"))
+    assert plan is not None and plan["gemm_cus"] > 0 and plan["mlp_gemm_cus"] > 0
+    y0, r0, _, layers, _, _ = run_stack(1000, "overlap", gemm_cus=plan["gemm_cus"],
+                                        mlp_gemm_cus=plan["mlp_gemm_cus"])
+    for layer in layers:   # attention of both splits, then the MLP of both splits
+        assert layer.budgets == [plan["gemm_cus"]] * 2 + [plan["mlp_gemm_cus"]] * 2
     y1, r1, _, layers, _, _ = run_stack(1000, "overlap")
     assert all(layer.budgets == [None] * 4 for layer in layers)
     assert torch.equal(y0, y1) and torch.equal(r0, r1)

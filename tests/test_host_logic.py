@@ -186,6 +186,28 @@ def test_weave_config_table_and_plan():
                                           "mlp_ctas": 4, "gemm_cus": 0}
 
 
+@pytest.mark.parametrize("name", ["llama_config_4", "llama_config_8", "mixtral_config_8", "qwen2_config_4",
+                                  "qwen2_config_8"])
+def test_every_reference_model_has_a_tuned_table(name):
+    """The reference ships five tables (vllm/tokenweave_configs/*.json); each has a
+    counterpart measured on MI355X with the same token counts, the reference's three
+    keys, the GEMM budgets and the measured overlap flag, and plans from it."""
+    cfg = tw.load_config(f"tokenweave_configs/{name}.json")
+    assert sorted(cfg) == [1024, 2048, 4096, 8192, 16384, 32768, 65536]
+    cus = 256
+    for n, e in cfg.items():
+        assert {"attention_ctas", "mlp_ctas", "split_offset", "gemm_cus", "mlp_gemm_cus", "overlap"} <= set(e)
+        assert e["overlap"] in (0, 1) and e["split_offset"] in (0, 256)
+        assert all(0 <= e[k] <= cus for k in ("attention_ctas", "mlp_ctas", "gemm_cus", "mlp_gemm_cus"))
+        plan = tw.weave_plan(n, cfg)
+        if e["overlap"]:
+            assert plan["split_size"] == n // 2 + e["split_offset"] and plan["rest_size"] == n - plan["split_size"]
+            assert plan["gemm_cus"] == e["gemm_cus"] and plan["mlp_gemm_cus"] == e["mlp_gemm_cus"]
+        else:
+            assert plan is None
+    assert cfg[65536]["overlap"] == 1, "long prefill chunks overlap on MI355X"
+
+
 def test_bind_checks_arguments_at_bind_time():
     import tokenweave_amd._custom_ops as ops
     x = torch.zeros(4, 64, dtype=torch.bfloat16)

@@ -25,11 +25,11 @@ from .layernorm import RMSNorm
 @lru_cache(maxsize=None)
 def load_config(config_path: str = "tokenweave_configs/llama_config_8.json") -> Dict[int, Dict[str, int]]:
     """Per-model weave table: token count -> {"attention_ctas", "mlp_ctas", "split_offset",
-    "gemm_cus"}.  Same file layout and loader contract as the reference
+    "gemm_cus", "mlp_gemm_cus", "overlap"}.  Same file layout and loader contract as the reference
     (tokenweave_utils.py:10-21, vllm/tokenweave_configs/*.json): JSON object with
     string token-count keys, returned with integer keys and cached per path.
     `*_ctas` is the MAX_CTAS given to the fused norm of the attention / MLP stage (0 =
-    one workgroup per row), `gemm_cus` the compute-unit budget of the GEMM it overlaps
+    one workgroup per row), `gemm_cus` / `mlp_gemm_cus` the compute-unit budget of the GEMM it overlaps
     with — the knob that matters on MI355X, where a GEMM workgroup and a norm workgroup
     cannot share a compute unit.  Relative paths resolve against this package."""
     base_dir = os.path.dirname(os.path.abspath(__file__))
@@ -60,9 +60,13 @@ def weave_plan(num_tokens: int, config: Dict[int, Dict[str, int]],
     if not entry.get("overlap", 1):
         return None
     split = min(tokenweave_split_size(num_tokens, entry.get("split_offset", 0)), num_tokens)
-    return {"split_size": split, "rest_size": num_tokens - split,
+    gemm_cus = entry.get("gemm_cus", 0)
+    plan = {"split_size": split, "rest_size": num_tokens - split,
             "attention_ctas": entry.get("attention_ctas", 0), "mlp_ctas": entry.get("mlp_ctas", 0),
-            "gemm_cus": entry.get("gemm_cus", 0)}
+            "gemm_cus": gemm_cus}
+    if "mlp_gemm_cus" in entry:
+        plan["mlp_gemm_cus"] = entry["mlp_gemm_cus"]
+    return plan
 
 
 class PartialsBuffer:
@@ -307,6 +311,7 @@ def tokenweave_overlap(
     mlp_fn: Optional[Callable] = None,
     all_ranks: bool = False,
     gemm_cus: int = 0,
+    mlp_gemm_cus: Optional[int] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """One decoder layer under the TokenWeave schedule (reference
     tokenweave_utils.py:175-340, same arguments and the same order of hand-offs):
@@ -322,8 +327,9 @@ def tokenweave_overlap(
     zeroed residual (residual <- sum of the partials, x <- norm of it).
     The last layer normalises split 1 after its MLP on the current stream (:327-339).
 
-    `gemm_cus` (no counterpart in the reference; `weave_plan(...)["gemm_cus"]`) is the
-    compute-unit budget of the GEMMs that run beside a norm: when non-zero it is handed to
+    `gemm_cus` / `mlp_gemm_cus` (no counterpart in the reference; `weave_plan(...)`) are the
+    compute-unit budgets of the GEMMs that run beside a norm (`mlp_gemm_cus` defaults to
+    `gemm_cus`): when non-zero they are handed to
     `self.self_attn(..., gemm_cus=)` and `mlp_fn(hidden_states, gemm_cus=)`, which pass it as
     `max_cus` to their row-parallel output projection (`ops.gemm_bf16_nt` /
     `ops.gemm_bf16_nt_partials`) so that the norm's workgroups find free compute units.  On
@@ -346,6 +352,8 @@ def tokenweave_overlap(
     rows_2 = _shard_rows(hidden_states_2.shape[0], rank, world_size, all_ranks)
 
     budget = {"gemm_cus": gemm_cus} if gemm_cus else {}
+    mlp_cus = gemm_cus if mlp_gemm_cus is None else mlp_gemm_cus
+    mlp_budget = {"gemm_cus": mlp_cus} if mlp_cus else {}
 
     def norm(layernorm, split, max_ctas):
         hs, res, blpr, off, rows = ((hidden_states_1, residual_1, blpr_1, 0, rows_1) if split == 0 else
@@ -381,14 +389,14 @@ def tokenweave_overlap(
         norm(self.post_attention_layernorm, 1, MAX_CTAS_MLP)
 
     with torch.cuda.stream(current_stream):
-        mlp_fn(hidden_states_1, **budget)
+        mlp_fn(hidden_states_1, **mlp_budget)
         current_stream.wait_stream(copy_stream)
     with torch.cuda.stream(copy_stream):
         copy_stream.wait_stream(current_stream)
         norm(next_layer_norm, 0, MAX_CTAS_MLP)
 
     with torch.cuda.stream(current_stream):
-        mlp_fn(hidden_states_2, **budget)
+        mlp_fn(hidden_states_2, **mlp_budget)
         current_stream.wait_stream(copy_stream)
 
     if layer_id == end_layer - 1:

@@ -94,6 +94,8 @@ def parse_args():
     ap.add_argument("--sweep", action="store_true", help="also time every configuration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-weave", action="store_true", help="leave the config 5 weave block out of the line")
+    ap.add_argument("--gemm-only", action="store_true",
+                    help="time only config 5's producer GEMM, one partial and all eight (for profiling)")
     ap.add_argument("--weave-only", action="store_true",
                     help="time only the GEMM + norm weave of config 5 and print its figures (for profiling)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -650,6 +652,33 @@ def time_weave(device, form="eight_partials", gemm_caps=(128,), norm_cap=0, step
     return {k: (round(v, 4) if isinstance(v, float) else v) for k, v in out.items()}
 
 
+def time_gemm_only(device, steps=200):
+    """Config 5's producer GEMM by itself, both forms, for profiling: [2458, 1024] x [8192, 1024]^T
+    into rotating staging buffers, `steps` launches of one partial and steps / 4 of all eight."""
+    import torch
+    from tokenweave_amd import _custom_ops as ops
+    from tokenweave_amd import workloads as wl
+    stream = torch.cuda.current_stream()
+    out = {}
+    for form, P, R, n in (("one_partial", 1, 8, steps), ("eight_partials", 8, 4, max(10, steps // 4))):
+        gs = wl.make_partials_gemm_inputs(P, device=device)
+        Ta, K = gs[0].a.shape
+        N = gs[0].b.shape[0]
+        stages = [torch.zeros((P, Ta, N), dtype=torch.bfloat16, device=device) for _ in range(R)]
+        if P == 1:
+            calls = [ops.bind_gemm_bf16_nt(stages[i][0], gs[0].a, gs[0].b) for i in range(R)]
+        else:
+            calls = [ops.bind_gemm_bf16_nt_partials([stages[i][p] for p in range(P)], [g.a for g in gs],
+                                                    [g.b for g in gs]) for i in range(R)]
+        us = event_time(lambda i: calls[i % R](stream), n, stream, warm=10, regions=3)
+        flops = 2.0 * P * Ta * N * K
+        out[form] = {"us": round(us, 2), "tflops": round(flops / us / 1e6, 1),
+                     "mfma_util": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        del calls, stages, gs
+        torch.cuda.empty_cache()
+    return out
+
+
 def weave_block(device, steps):
     """Both forms of config 5 for the JSON line."""
     caps = (128, 160, 192, 224, 240)
@@ -687,6 +716,9 @@ def main():
     if args.timeline:
         print(json.dumps({"timeline": time_timeline(cfg, device), "arrivals": time_arrivals(cfg, device)}),
               flush=True)
+        return
+    if args.gemm_only:
+        print(json.dumps({"c5_gemm": time_gemm_only(device, min(args.steps, 200))}), flush=True)
         return
     if args.weave_only:
         print(json.dumps({"weave": weave_block(device, min(args.steps, 200))}), flush=True)

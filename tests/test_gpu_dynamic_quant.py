@@ -159,16 +159,29 @@ def test_partials_against_checker_and_grid_cap_invariance(oracle, T, add_residua
 
 
 @pytest.mark.parametrize("quant_dtype", [torch.int8, FP8])
-def test_full_size_properties(quant_dtype):
-    """8192 x 6144, P = 8 (too long for the CPU checker): every row uses the whole
-    code range, dequantised codes reproduce the unquantised op's output to the
-    format's precision, the residual equals the unquantised op's."""
+def test_full_size_against_checker_on_sampled_rows_and_properties(oracle, quant_dtype):
+    """8192 x 6144, P = 8.  512 rows spread over the launch (the first and last rows, a
+    stride through the middle) are compared with the CPU checker code for code; over all
+    rows: every row uses the whole code range, dequantised codes reproduce the
+    unquantised op's output to the format's precision, the residual equals the
+    unquantised op's."""
     cfg = wl.C4
     inp = wl.make_norm_inputs(cfg, DEV)
     out = torch.empty(cfg.T, cfg.H, dtype=quant_dtype, device=DEV)
     scales = torch.empty(cfg.T, 1, dtype=torch.float32, device=DEV)
     res = inp.residual.clone()
     ops.reduce_add_rms_norm_dynamic_per_token_quant(inp.partials, out, scales, res, inp.weight, cfg.eps)
+    torch.cuda.synchronize()
+    rows = torch.unique(torch.cat([torch.arange(0, 64), torch.arange(cfg.T - 64, cfg.T),
+                                   torch.arange(64, cfg.T - 64, (cfg.T - 128) // 384)[:384]])).to(DEV)
+    assert rows.numel() >= 500
+    kind = oracle.QUANT_FP8 if quant_dtype == FP8 else oracle.QUANT_INT8
+    r_np = to_bits(inp.residual[rows])
+    want, want_scales = oracle.rms_norm_dynamic_per_token_quant([to_bits(p[rows]) for p in inp.partials],
+                                                                to_bits(inp.weight), cfg.eps, kind, r=r_np)
+    assert np.array_equal(to_bits(res[rows]), r_np), "residual differs from the checker on the sampled rows"
+    assert_codes_and_scales(out[rows], scales[rows], torch.from_numpy(want).view(quant_dtype),
+                            torch.from_numpy(want_scales), quant_dtype, "C4 sampled rows")
     y = torch.empty_like(inp.residual)
     res2 = inp.residual.clone()
     ops.reduce_add_rms_norm(inp.partials, y, res2, inp.weight, cfg.eps)

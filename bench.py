@@ -759,7 +759,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
         log(f"[bench] cpu_baseline {out['cpu_baseline']}")
     if not args.no_weave:
-        out["weave"] = weave_block(device, 40)
+        out["weave"] = weave_block(device, 100)
         log(f"[bench] weave {out['weave']}")
     if args.calibration_copy:
         calibration_copies(device)

@@ -118,7 +118,7 @@ class NormRunner:
     ctypes call per launch) for each input set, so that the host enqueues a step
     faster than the GPU runs it."""
 
-    def __init__(self, cfg, nsets, max_ctas, device, epilogue="bf16"):
+    def __init__(self, cfg, nsets, max_ctas, device, epilogue="bf16", split=None):
         import torch
         from tokenweave_amd import _custom_ops as ops
         from tokenweave_amd import _lib
@@ -130,7 +130,7 @@ class NormRunner:
             if epilogue == "bf16":
                 # y lands on this rank's staging rows (rank 0)
                 op = ops.bind_reduce_add_rms_norm(inp.partials, inp.partials[0], inp.residual, inp.weight,
-                                                  cfg.eps, max_ctas or None)
+                                                  cfg.eps, max_ctas or None, split=split)
             else:
                 op = self._bind_quant(ops, L, torch, cfg, epilogue, inp, max_ctas, device)
             op()  # one launch up front: a bad argument fails here, not in the timed loop
@@ -178,7 +178,7 @@ LEAD_IN = 40        # untimed launches ahead of an event bracket (the bracket st
 
 
 def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16", regions=REGIONS, preroll_ms=PREROLL_MS,
-              lead_in=LEAD_IN):
+              lead_in=LEAD_IN, split=None):
     """After an untimed pre-roll and `warmup` warm-up launches, times `regions` regions of
     exactly `steps` back-to-back launches twice over: by the wall clock between two device
     synchronisations (ms_per_step, gbps), and by HIP events on the launch stream around
@@ -189,7 +189,7 @@ def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16", regions=REG
     free, _ = torch.cuda.mem_get_info()
     set_bytes = (cfg.P + 1) * cfg.T * cfg.H * 2 + cfg.H * 2
     nsets = max(2, min(nsets, int(free * 0.6) // (set_bytes * 3)))  # fp32 staging while generating
-    runner = NormRunner(cfg, nsets, max_ctas, device, epilogue)
+    runner = NormRunner(cfg, nsets, max_ctas, device, epilogue, split)
     stream = torch.cuda.current_stream()
     it = 0
     preroll_steps = max(warmup, int(preroll_ms * 1e3 / max(2.0, cfg.bytes / 6e6)))
@@ -771,7 +771,12 @@ def main():
             steps = max(50, min(2000, int(0.02 * 5e12 / c.bytes)))  # ~20 ms of kernel time
             r = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device, regions=5, preroll_ms=10.0)
             warm_us = time_norm_warm(c, steps, args.max_ctas, device) if c.bytes < (200 << 20) else None
+            one_wg = None
+            if c.P > 1 and c.T <= 48:   # decode sizes: the same call without the split-row kernel
+                one_wg = time_norm(c, steps, max(5, steps // 10), args.max_ctas, device, regions=5, preroll_ms=10.0,
+                                   split=False)["event_us_per_launch"]
             sweep[name] = {"P": c.P, "T": c.T, "H": c.H, "bytes": c.bytes,
+                           "kernel_us_one_workgroup_per_row": None if one_wg is None else round(one_wg, 3),
                            "us_per_call": round(r["ms_per_step"] * 1e3, 3),
                            "kernel_us": round(r["event_us_per_launch"], 3),
                            "kernel_us_cache_resident": None if warm_us is None else round(warm_us, 3),

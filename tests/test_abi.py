@@ -40,7 +40,8 @@ def test_header_cites_the_reference_interface_for_each_op():
     for cite in ("csrc/layernorm_kernels.cu:194-231", "csrc/torch_bindings.cpp:141-144",
                  "csrc/tokenweave_fused_kernels.cu:220-261", "csrc/torch_bindings.cpp:152-157",
                  "csrc/tokenweave_artifact_kernels.cu:717-754", "csrc/tokenweave_artifact_kernels.cu:772-813",
-                 "csrc/tokenweave_fused_kernels.cu:186-202", "vllm/model_executor/layers/linear.py:203-228"):
+                 "csrc/tokenweave_fused_kernels.cu:186-202", "vllm/model_executor/layers/linear.py:203-228",
+                 "1310-1321", "csrc/tokenweave_fused_kernels.cu:241-244"):
         assert cite in text, cite
 
 
@@ -92,6 +93,42 @@ def test_cta_entry_points_refuse_misaligned_or_odd_hidden_like_the_reference():
     assert "Invalid rank 2" in _lib.last_error()
     assert L.tw_fused_rs_ln_cta(ALIGNED, ALIGNED, ALIGNED, 0, 1024, 0, 2, 8, 1e-5, 4, 64, None) == _lib.TW_ERR_INVALID_ARGUMENT
     assert L.tw_fused_rs_ln_cta(ALIGNED, ALIGNED, ALIGNED, ALIGNED, 1024, 0, 17, 8, 1e-5, 4, 64, None) == _lib.TW_ERR_INVALID_ARGUMENT
+
+
+def test_workspace_and_static_workspace_entry_points_check_before_they_launch():
+    L = _lib.lib()
+    ptrs = (ctypes.c_void_p * 2)(ALIGNED, ALIGNED)
+    args = (ptrs, 2, ALIGNED, ALIGNED, ALIGNED, 4, 64, 0, 1e-5)
+    assert L.tw_reduce_add_rms_norm_ws(*args, ALIGNED, 100, None) == _lib.TW_ERR_INVALID_ARGUMENT
+    assert "workspace" in _lib.last_error() and str(_lib.TW_SPLIT_WORKSPACE_BYTES) in _lib.last_error()
+    assert L.tw_fused_rs_ln_ag_cta_ws(ALIGNED, ALIGNED, ALIGNED, ALIGNED, 1024, 0, 2, 0, 1e-5, 4, 64, ALIGNED, 100,
+                                      None) == _lib.TW_ERR_INVALID_ARGUMENT
+    assert L.tw_reduce_add_rms_norm_ws(ptrs, 2, ALIGNED, None, ALIGNED, 4, 64, 0, 1e-5, None, 0, None) == \
+        _lib.TW_ERR_INVALID_ARGUMENT
+    assert L.tw_reduce_add_rms_norm_ws(ptrs, 2, None, None, None, 0, 64, 0, 1e-5, None, 0, None) == _lib.TW_OK
+    # the static workspace holds TW_SPLIT_MAX_TOKENS rows: larger batches are refused up front
+    too_many = _lib.TW_SPLIT_MAX_TOKENS + 1
+    assert L.tw_reduce_add_rms_norm_noalloc(ptrs, 2, ALIGNED, ALIGNED, ALIGNED, too_many, 64, 0, 1e-5, None) == \
+        _lib.TW_ERR_INVALID_ARGUMENT
+    assert "exceeds" in _lib.last_error()
+    assert _lib.TW_SPLIT_WORKSPACE_BYTES == 256 * 384
+    text = open(HEADER).read()
+    assert "#define TW_SPLIT_MAX_TOKENS 256" in text and "(TW_SPLIT_MAX_TOKENS * 384)" in text
+
+
+def test_partials_producer_argument_checks():
+    L = _lib.lib()
+    vp = ctypes.c_void_p
+    three = (vp * 3)(ALIGNED, ALIGNED, ALIGNED)
+    assert L.tw_gemm_bf16_nt_partials(three, three, three, 0, 16, 64, 64, 64, 0, None) == _lib.TW_ERR_INVALID_ARGUMENT
+    assert L.tw_gemm_bf16_nt_partials(three, three, three, 17, 16, 64, 64, 64, 0, None) == _lib.TW_ERR_INVALID_ARGUMENT
+    assert L.tw_gemm_bf16_nt_partials(three, three, three, 3, 0, 64, 64, 64, 0, None) == _lib.TW_OK
+    assert L.tw_gemm_bf16_nt_partials(three, three, three, 3, 16, 64, 12, 64, 0, None) == _lib.TW_ERR_ALIGNMENT
+    bad = (vp * 3)(ALIGNED, None, ALIGNED)
+    assert L.tw_gemm_bf16_nt_partials(three, bad, three, 3, 16, 64, 64, 64, 0, None) == _lib.TW_ERR_INVALID_ARGUMENT
+    odd = (vp * 3)(ALIGNED, ALIGNED + 4, ALIGNED)
+    assert L.tw_gemm_bf16_nt_partials(odd, three, three, 3, 16, 64, 64, 64, 0, None) == _lib.TW_ERR_ALIGNMENT
+    assert L.tw_gemm_bf16_nt_partials(None, three, three, 3, 16, 64, 64, 64, 0, None) == _lib.TW_ERR_INVALID_ARGUMENT
 
 
 def test_gemm_argument_checks():

@@ -382,7 +382,8 @@ class BoundOp:
             _lib.check(rc)
 
 
-def _prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS, split=None):
+def _check_reduce_add_rms_norm(partials, out, residual, weight, MAX_CTAS):
+    """Argument checks of the pointer-list op; returns (ptrs, P, T, H, cap, device)."""
     P = len(partials)
     _require(1 <= P <= _lib.TW_MAX_PARTIALS,
              f"number of partials {P} not in [1, {_lib.TW_MAX_PARTIALS}]")
@@ -399,16 +400,7 @@ def _prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_C
             raise RuntimeError(f"partials[{i}] has shape {tuple(p.shape)}, expected {tuple(out.shape)}")
     _check_weight(weight, H, torch.bfloat16, dev)
     ptrs = (ctypes.c_void_p * P)(*[p.data_ptr() for p in partials])
-    cap = _cap(MAX_CTAS)
-    if _wants_split(T, cap) if split is None else split:
-        # decode-size batch: the split-row kernel, with a workspace of the op's own (a bound
-        # op may be launched on any stream, but not on two at once)
-        ws = torch.zeros(_lib.TW_SPLIT_WORKSPACE_BYTES, dtype=torch.uint8, device=dev)
-        args = (ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H, cap, epsilon,
-                ws.data_ptr(), ws.numel())
-        return _lib.lib().tw_reduce_add_rms_norm_ws, args, (list(partials), out, residual, weight, ws), dev
-    args = (ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H, cap, epsilon)
-    return _lib.lib().tw_reduce_add_rms_norm, args, (list(partials), out, residual, weight), dev
+    return ptrs, P, T, H, _cap(MAX_CTAS), dev
 
 
 def reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
@@ -416,25 +408,38 @@ def reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
                         MAX_CTAS: Optional[int] = None, split: Optional[bool] = None) -> None:
     """out <- RMSNorm(sum_p partials[p] + residual) * weight; residual <- the sum.
     `out` may be one of the partials.  Uncapped calls of at most TW_SPLIT_MAX_TOKENS rows
-    go through the split-row entry point (several workgroups per row, same bits);
-    `split=False` forces the one-workgroup-per-row kernel."""
-    fn, args, keep, dev = _prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS,
-                                                       False)
-    if (_wants_split(args[5], args[7]) if split is None else split):
-        idx = dev.index if dev.index is not None else torch.cuda.current_device()
-        with _on_device(out):
-            sp = _stream_ptr(out)
-            ws = split_workspace(idx, sp)
-            _lib.check(_lib.lib().tw_reduce_add_rms_norm_ws(*args, ws.data_ptr(), ws.numel(), sp))
-        return
-    BoundOp(fn, args, keep, dev)()
+    go through the split-row entry point (several workgroups per row where that pays, same
+    bits) with the workspace of the current stream; `split=False` forces the
+    one-workgroup-per-row kernel."""
+    ptrs, P, T, H, cap, dev = _check_reduce_add_rms_norm(partials, out, residual, weight, MAX_CTAS)
+    L = _lib.lib()
+    with _on_device(out):
+        sp = _stream_ptr(out)
+        if _wants_split(T, cap) if split is None else split:
+            ws = split_workspace(dev.index if dev.index is not None else torch.cuda.current_device(), sp)
+            rc = L.tw_reduce_add_rms_norm_ws(ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H,
+                                             cap, epsilon, ws.data_ptr(), ws.numel(), sp)
+        else:
+            rc = L.tw_reduce_add_rms_norm(ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H,
+                                          cap, epsilon, sp)
+    if rc:
+        _lib.check(rc)
 
 
 def bind_reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
                              residual: torch.Tensor, weight: torch.Tensor, epsilon: float,
                              MAX_CTAS: Optional[int] = None, split: Optional[bool] = None) -> BoundOp:
-    """`reduce_add_rms_norm` with the checks done now and the launch deferred."""
-    return BoundOp(*_prepare_reduce_add_rms_norm(partials, out, residual, weight, epsilon, MAX_CTAS, split))
+    """`reduce_add_rms_norm` with the checks done now and the launch deferred.  A bound op
+    of a decode-size batch owns its split-row workspace: it may be launched on any stream,
+    but not on two at once."""
+    ptrs, P, T, H, cap, dev = _check_reduce_add_rms_norm(partials, out, residual, weight, MAX_CTAS)
+    keep = [list(partials), out, residual, weight]
+    args = (ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H, cap, epsilon)
+    if _wants_split(T, cap) if split is None else split:
+        ws = torch.zeros(_lib.TW_SPLIT_WORKSPACE_BYTES, dtype=torch.uint8, device=dev)
+        keep.append(ws)
+        return BoundOp(_lib.lib().tw_reduce_add_rms_norm_ws, args + (ws.data_ptr(), ws.numel()), keep, dev)
+    return BoundOp(_lib.lib().tw_reduce_add_rms_norm, args, keep, dev)
 
 
 def split_segments(num_tokens: int, hidden_size: int, MAX_CTAS: Optional[int] = None) -> int:

@@ -411,6 +411,10 @@ def time_timeline(cfg, device, launches=200):
         "stores_acknowledged_after_y_issue_us": rows_stat(st[:, :, 5] - st[:, :, 4]),
         "row_end_after_first_row_us": rows_stat(rel[:, :, 5]),
         "rows_per_xcc_first_launch": [int((xcc[0] == x).sum()) for x in range(8)],
+        "median_row_begin_by_xcc_us": [round(med(rel[:, :, 0][xcc == x]), 2) if (xcc == x).any() else None
+                                       for x in range(8)],
+        "median_loads_returned_by_xcc_us": [round(med(rel[:, :, 1][xcc == x]), 2) if (xcc == x).any() else None
+                                            for x in range(8)],
         "median_row_end_by_xcc_us": [round(med(rel[:, :, 5][xcc == x]), 2) if (xcc == x).any() else None
                                      for x in range(8)],
     }

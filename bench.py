@@ -74,6 +74,8 @@ def bench_lib():
         L.twb_trace_stream_rows.argtypes = [ctypes.POINTER(vp), vp, i64, i64, vp]
         L.twb_empty.argtypes = [ci, ci, vp]
         L.twb_trace_reduce_add_rms_norm.argtypes = [ctypes.POINTER(vp), ci, vp, vp, vp, i64, i64, ci, f32, vp, vp]
+        L.twb_gemm_loop.argtypes = [ci, ci, i64, vp, vp, vp, ci, vp]
+        L.twb_lds_read_rate.argtypes = [ci, ci, ci, vp, vp, vp, ci, vp]
         L.tw_last_error.restype = ctypes.c_char_p
         _BENCH_LIB = L
     return _BENCH_LIB
@@ -96,6 +98,9 @@ def parse_args():
     ap.add_argument("--no-weave", action="store_true", help="leave the config 5 weave block out of the line")
     ap.add_argument("--gemm-only", action="store_true",
                     help="time only config 5's producer GEMM, one partial and all eight (for profiling)")
+    ap.add_argument("--gemm-limits", action="store_true",
+                    help="time the GEMM's k loop assembled from its parts (MFMAs, LDS fragment reads, operand "
+                         "slabs global -> LDS) on L2-resident operands, and the LDS read rate, and print them")
     ap.add_argument("--weave-only", action="store_true",
                     help="time only the GEMM + norm weave of config 5 and print its figures (for profiling)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -683,6 +688,63 @@ def time_gemm_only(device, steps=200):
     return out
 
 
+def time_gemm_limits(device):
+    """What the big GEMM kernel's k loop can reach by itself on this GPU: the loop of the 320 x 256 tile
+    put together from its parts, every compute unit busy, operands served by the L2s, no tile prologue
+    or epilogue.  TFLOP/s from HIP events around the launch; cycles and clock from the kernel's own stamps.
+    Also the rate at which 1 .. 16 waves of a compute unit get the loop's 16-byte LDS reads through."""
+    import numpy as np
+    import torch
+    L = bench_lib()
+    stream = torch.cuda.current_stream()
+    sp = stream.cuda_stream
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    window = 4 << 20
+    src = torch.randint(0, 255, (8 * window + (128 << 10),), dtype=torch.uint8, device=device)
+    stamps = torch.zeros((cus, 2), dtype=torch.int64, device=device)
+    sink = torch.zeros(1024, dtype=torch.float32, device=device)
+    slabs = 8192
+    flops = cus * 8 * slabs * 40 * 32768.0   # 8 waves x 40 MFMAs of 32 x 32 x 16 per slab
+    loop = {}
+    for name, parts in (("mfma", 0), ("mfma+lds_reads", 1), ("mfma+slab_loads", 2), ("full_loop", 3),
+                        ("full_loop_loads_spread", 7)):
+        ms = []
+        for _ in range(4):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            bench_check(L.twb_gemm_loop(slabs, parts, window, src.data_ptr(), stamps.data_ptr(), sink.data_ptr(),
+                                        cus, sp))
+            e1.record(stream)
+            torch.cuda.synchronize()
+            ms.append(e0.elapsed_time(e1))
+        st = stamps.cpu().numpy().astype(np.float64)
+        cyc, wall_us = float(np.median(st[:, 0])), float(np.median(st[:, 1])) / 100.0
+        t = sorted(ms[1:])[1] * 1e-3
+        loop[name] = {"cycles_per_slab": round(cyc / slabs), "mfma_issue_share": round(2560.0 * slabs / cyc, 3),
+                      "shader_clock_ghz": round(cyc / wall_us / 1e3, 2), "tflops": round(flops / t / 1e12, 1),
+                      "share_of_2.5_pflops": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 3)}
+    lds = {}
+    iters = 2000
+    cyc_out = torch.zeros(cus, dtype=torch.int64, device=device)
+    usink = torch.zeros(1024, dtype=torch.int32, device=device)
+    for waves in (1, 2, 4, 8, 16):
+        for dma in (0, 1):
+            for _ in range(2):
+                bench_check(L.twb_lds_read_rate(iters, waves, dma, src.data_ptr(), cyc_out.data_ptr(), usink.data_ptr(),
+                                                cus, sp))
+                torch.cuda.synchronize()
+            cyc = float(np.median(cyc_out.cpu().numpy()))
+            lds[f"waves{waves}" + ("+slab_loads" if dma else "")] = {
+                "read_bytes_per_cycle": round(waves * iters * 28 * 1024 / cyc, 1),
+                "cycles_per_read_per_wave": round(cyc / (iters * 28), 1)}
+    return {"definitions": "loop: the k loop of the 320 x 256 x 64 tile (8 waves, 40 MFMAs of 32 x 32 x 16 and 28 "
+                           "16-byte LDS reads per wave and slab, 72 KiB per slab global -> LDS) with wait + barrier "
+                           "per slab, on all compute units, operands in a 4 MiB window per XCD; mfma_issue_share "
+                           "= 2560 MFMA cycles per slab / measured cycles per slab; lds: 16-byte reads with the "
+                           "fragment addressing",
+            "loop": loop, "lds_read_rate": lds}
+
+
 def weave_block(device, steps):
     """Both forms of config 5 for the JSON line."""
     caps = (128, 160, 192, 224, 240)
@@ -723,6 +785,9 @@ def main():
         return
     if args.gemm_only:
         print(json.dumps({"c5_gemm": time_gemm_only(device, min(args.steps, 200))}), flush=True)
+        return
+    if args.gemm_limits:
+        print(json.dumps({"gemm_limits": time_gemm_limits(device)}), flush=True)
         return
     if args.weave_only:
         print(json.dumps({"weave": weave_block(device, min(args.steps, 200))}), flush=True)

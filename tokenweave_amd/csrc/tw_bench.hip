@@ -9,7 +9,11 @@
 //    norm kernel's exact traffic (nine streams read, two written in place) without
 //    arithmetic, reduction or barrier, a plain copy with default cache policy whose
 //    traffic is known exactly (hardware counters are scaled against it), and an empty
-//    kernel (launch-to-launch floor).
+//    kernel (launch-to-launch floor);
+//  * the main loop of the big GEMM kernel put together from its parts (MFMAs, fragment
+//    reads from LDS, operand slabs global -> LDS, the barrier per k-slab) on operands that
+//    stay in the L2s, and the rate at which waves get 16-byte LDS reads through: what the
+//    loop itself can reach on this machine, apart from tile prologue and epilogue.
 #define TW_TRACE 1
 #include "tw_api.hip"
 #include "tw_gemm.hip"
@@ -140,6 +144,142 @@ __global__ __launch_bounds__(256) void copy16_kernel(uint4* __restrict__ dst, co
 
 __global__ void empty_kernel() {}
 
+
+// The k loop of gemm_bf16_nt_big_kernel<5, 2> (eight waves, 160 x 64 wave tiles, 320 x 256 x 64
+// slabs, two LDS stages) assembled from switchable parts; the arithmetic result is
+// meaningless.  parts bit 0: fragment reads from LDS (else the MFMAs reuse their first
+// operands); bit 1: the slab loads global -> LDS (from a `window`-byte region per XCD, so
+// the L2s serve them); bit 2: issue the slab's loads over the four k-steps instead of at
+// the slab's head.  Every variant keeps the wait + barrier per slab, which also keeps the
+// two waves of a SIMD in step, so that wave 0's clock stamps stand for the workgroup.
+// out[2 b] = shader-clock cycles, out[2 b + 1] = wall clock (10 ns) of workgroup b.
+__global__ __launch_bounds__(512) void gemm_loop_kernel(int slabs, int parts, uint32_t window, const uint8_t* src,
+                                                        long long* out, float* sink) {
+  constexpr int TM = 5, TN = 2, STAGE = (320 + 256) * 128, LOADS = 9;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const bool reads = parts & 1, loads = parts & 2, spread = parts & 4;
+  for (int i = threadIdx.x; i < 2 * STAGE / 4; i += blockDim.x)
+    reinterpret_cast<uint32_t*>(lds)[i] = 0x3c003c00u + (i & 3);
+  __syncthreads();
+  uint32_t roff[4];
+  for (int kk = 0; kk < 4; ++kk) roff[kk] = l32 * 128 + ((((kk << 1) | lhi) ^ ((l32 >> 1) & 7)) << 4);
+  const uint8_t* pa = lds + (wave >> 2) * (32 * TM) * 128;
+  const uint8_t* pb = lds + 320 * 128 + (wave & 3) * (32 * TN) * 128;
+  const __amdgpu_buffer_rsrc_t d = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(src) + (size_t)(blockIdx.x & 7) * window, 0, window, 0x00020000);
+  tw::f32x16_t acc[TM][TN];
+  for (int i = 0; i < TM; ++i)
+    for (int j = 0; j < TN; ++j)
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  tw::bf16x8_t fa[2][TM], fb[2][TN];
+  for (int i = 0; i < TM; ++i)
+    fa[0][i] = fa[1][i] = __builtin_bit_cast(tw::bf16x8_t, *reinterpret_cast<const uint4*>(pa + i * 4096 + roff[0]));
+  for (int j = 0; j < TN; ++j)
+    fb[0][j] = fb[1][j] = __builtin_bit_cast(tw::bf16x8_t, *reinterpret_cast<const uint4*>(pb + j * 4096 + roff[0]));
+  __syncthreads();
+  const long long t0 = wall_clock64();
+  const long long c0 = __builtin_readcyclecounter();
+  for (int s = 0; s < slabs; ++s) {
+    const int stage = s & 1;
+    // a different slab-sized piece of the window per workgroup and slab
+    uint32_t base = (uint32_t)(((blockIdx.x >> 3) * STAGE + s * STAGE * 7) & (window - 1)) & ~1023u;
+    if (base > window - STAGE) base = window - STAGE;  // the whole slab lies inside the window
+    uint8_t* dst = lds + (stage ^ 1) * STAGE + wave * LOADS * 1024;
+    const uint8_t* qa = pa + stage * STAGE;
+    const uint8_t* qb = pb + stage * STAGE;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const int cur = kk & 1, nxt = cur ^ 1;
+      if (loads) {
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j)
+          if (spread ? (j * 4) / LOADS == kk : kk == 0)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(d, (tw::lds_void_t*)(dst + j * 1024), 16,
+                                                     (uint32_t)(lane * 16 + (wave * LOADS + j) * 1024), base, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < (TM + 1) / 2; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (reads) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          fa[nxt][i] = __builtin_bit_cast(tw::bf16x8_t,
+                                          *reinterpret_cast<const uint4*>(qa + i * 4096 + roff[(kk + 1) & 3]));
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          fb[nxt][j] = __builtin_bit_cast(tw::bf16x8_t,
+                                          *reinterpret_cast<const uint4*>(qb + j * 4096 + roff[(kk + 1) & 3]));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = (TM + 1) / 2; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+  const long long c1 = __builtin_readcyclecounter();
+  const long long t1 = wall_clock64();
+  float t = 0.0f;
+  for (int i = 0; i < TM; ++i)
+    for (int j = 0; j < TN; ++j)
+      for (int e = 0; e < 16; ++e) t += acc[i][j][e];
+  if (t == 12345.678f) sink[threadIdx.x] = t;  // keeps the MFMAs alive; never true
+  if (threadIdx.x == 0) {
+    out[blockIdx.x * 2] = c1 - c0;
+    out[blockIdx.x * 2 + 1] = t1 - t0;
+  }
+}
+
+// 16-byte LDS reads with the GEMM's fragment addressing, 28 per wave and iteration (one
+// k-slab's worth), by blockDim / 64 waves; dma: each wave also brings nine 1 KiB pieces
+// global -> LDS per iteration (the slab loads).  out[b] = shader-clock cycles of workgroup b.
+__global__ __launch_bounds__(1024) void lds_read_rate_kernel(int iters, int dma, const uint8_t* src, long long* out,
+                                                             uint32_t* sink) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int l32 = lane & 31, lhi = lane >> 5;
+  for (int i = threadIdx.x; i < 147456 / 4; i += blockDim.x) reinterpret_cast<uint32_t*>(lds)[i] = i;
+  uint32_t roff[4];
+  for (int kk = 0; kk < 4; ++kk) roff[kk] = l32 * 128 + ((((kk << 1) | lhi) ^ ((l32 >> 1) & 7)) << 4);
+  const uint8_t* base = lds + (wave % 8) * 8192;
+  const __amdgpu_buffer_rsrc_t d = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(src), 0, 1u << 20, 0x00020000);
+  uint4 acc = make_uint4(0, 0, 0, 0);
+  __syncthreads();
+  const long long c0 = __builtin_readcyclecounter();
+  for (int it = 0; it < iters; ++it) {
+    if (dma && wave < 8) {
+#pragma unroll
+      for (int j = 0; j < 9; ++j)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(d, (tw::lds_void_t*)(lds + 73728 + (wave * 9 + j) * 1024), 16,
+                                                 (uint32_t)(lane * 16 + (wave * 9 + j) * 1024), 0, 0, 0);
+    }
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+#pragma unroll
+      for (int f = 0; f < 7; ++f) {
+        const uint4 v = *reinterpret_cast<const uint4*>(base + f * 4096 + roff[kk]);
+        acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w;
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+  const long long c1 = __builtin_readcyclecounter();
+  if (threadIdx.x == 0) out[blockIdx.x] = c1 - c0;
+  if (acc.x == 0x12345u && acc.y == 7u) sink[threadIdx.x] = acc.z + acc.w;  // never true for the fill above
+}
+
 }  // namespace twb
 
 extern "C" {
@@ -225,6 +365,38 @@ TW_API int twb_trace_reduce_add_rms_norm(const void* const* partials, int num_pa
     return tw::set_error(TW_ERR_LAUNCH, "trace: could not set the trace pointer");
   return tw::run_row_norm("trace_reduce_add_rms_norm", partials, num_partials, y, residual, nullptr, weight,
                           nullptr, num_tokens, hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true, stream);
+}
+
+
+static int bench_lds_limit(const void* fn, int bytes) {
+  return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess ? TW_OK
+             : tw::set_error(TW_ERR_LAUNCH, "the device refused %d bytes of LDS", bytes);
+}
+
+// The GEMM's k loop from its parts (see gemm_loop_kernel).  src: 8 * window bytes of device
+// memory, window a power of two >= 128 KiB; out: 2 * grid int64; sink: 512 floats.
+TW_API int twb_gemm_loop(int slabs, int parts, int64_t window, const void* src, void* out, void* sink, int grid,
+                         void* stream) {
+  if (slabs < 1 || grid < 1 || !src || !out || !sink || window < (128 << 10) || window > (1ll << 30) ||
+      (window & (window - 1)))
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "gemm_loop: bad argument");
+  if (int rc = bench_lds_limit(reinterpret_cast<const void*>(twb::gemm_loop_kernel), 147456)) return rc;
+  tw::launch_kernel(twb::gemm_loop_kernel, dim3((unsigned)grid), dim3(512), 147456, static_cast<hipStream_t>(stream),
+                    slabs, parts, (uint32_t)window, static_cast<const uint8_t*>(src), static_cast<long long*>(out),
+                    static_cast<float*>(sink));
+  return tw::finish_launch("gemm_loop");
+}
+
+// src: 1 MiB of device memory; out: grid int64; sink: 1024 uint32.
+TW_API int twb_lds_read_rate(int iters, int waves, int dma, const void* src, void* out, void* sink, int grid,
+                             void* stream) {
+  if (iters < 1 || waves < 1 || waves > 16 || grid < 1 || !src || !out || !sink)
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "lds_read_rate: bad argument");
+  if (int rc = bench_lds_limit(reinterpret_cast<const void*>(twb::lds_read_rate_kernel), 147456)) return rc;
+  tw::launch_kernel(twb::lds_read_rate_kernel, dim3((unsigned)grid), dim3((unsigned)waves * 64), 147456,
+                    static_cast<hipStream_t>(stream), iters, dma, static_cast<const uint8_t*>(src),
+                    static_cast<long long*>(out), static_cast<uint32_t*>(sink));
+  return tw::finish_launch("lds_read_rate");
 }
 
 }  // extern "C"

@@ -344,10 +344,14 @@ template <typename E, int NP, int VPT, int MAXNT, bool HAS_RES, bool COPY, int Q
 __device__ __forceinline__ void row_norm_vec_body(
     const PartialPtrs& parts, int np_rt, void* y_out, void* residual, void* copy_out,
     const void* __restrict__ weight, const float* __restrict__ quant_scale,
-    float* __restrict__ row_scales, float eps, int num_tokens, int vec_per_row, float hidden,
+    float* __restrict__ row_scales, float eps, int num_tokens, int vec_per_row, float hidden, int nt, int grid,
     float (*slots)[kMaxChunks], float (*max_slots)[16]) {
   constexpr bool FP8 = Q == kQStaticFp8;
-  const int nt = blockDim.x;
+  // nt = lanes per workgroup and grid = workgroups come as kernel arguments, and the
+  // launcher never starts more workgroups than there are rows (the row loop tests at
+  // its end): read from the dispatch packet's hidden arguments (blockDim, gridDim), and
+  // with a test of the row count ahead of the first row, the kernel would make two more
+  // dependent memory round trips before the row's first load can go out.
   const int nwaves = nt >> 6;
   const int nchunks = (vec_per_row + 63) >> 6;  // <= VPT * nwaves
   const int np = NP > 0 ? NP : np_rt;
@@ -363,7 +367,8 @@ __device__ __forceinline__ void row_norm_vec_body(
   if (Q != kQNone && quant_scale) qparam = *quant_scale;
 
   int phase = 0;
-  for (int row = blockIdx.x; row < num_tokens; row += gridDim.x, phase ^= 1) {
+  int row = blockIdx.x;
+  do {
     float s[VPT][8];
     uint4 first[VPT];
     uint4 wv[VPT];     // the weight row is fetched per token row, behind the row's own loads
@@ -501,43 +506,45 @@ __device__ __forceinline__ void row_norm_vec_body(
           store8(dy, off[k] / 2, quant4_fp8_div(n[0], n[1], n[2], n[3], scale),
                  quant4_fp8_div(n[4], n[5], n[6], n[7], scale));
       }
-      continue;
-    }
-    const float scale_inv = 1.0f / qparam;
+    } else {
+      const float scale_inv = 1.0f / qparam;
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) {
-      float r[8], w[8];
-      unpack8e<E>(rnew[k], r);
-      unpack8e<E>(wv[k], w);
-      uint4 o;
-      o.x = Pk<E>::pack(r[0] * inv * w[0], r[1] * inv * w[1]);
-      o.y = Pk<E>::pack(r[2] * inv * w[2], r[3] * inv * w[3]);
-      o.z = Pk<E>::pack(r[4] * inv * w[4], r[5] * inv * w[5]);
-      o.w = Pk<E>::pack(r[6] * inv * w[6], r[7] * inv * w[7]);
-      if (FP8) {
-        float y[8];
-        unpack8e<E>(o, y);
-        store8(dy, off[k] / 2, quant4_fp8(y[0], y[1], y[2], y[3], scale_inv),
-               quant4_fp8(y[4], y[5], y[6], y[7], scale_inv));
-      } else {
-        store16(dy, off[k], o);
+      for (int k = 0; k < VPT; ++k) {
+        float r[8], w[8];
+        unpack8e<E>(rnew[k], r);
+        unpack8e<E>(wv[k], w);
+        uint4 o;
+        o.x = Pk<E>::pack(r[0] * inv * w[0], r[1] * inv * w[1]);
+        o.y = Pk<E>::pack(r[2] * inv * w[2], r[3] * inv * w[3]);
+        o.z = Pk<E>::pack(r[4] * inv * w[4], r[5] * inv * w[5]);
+        o.w = Pk<E>::pack(r[6] * inv * w[6], r[7] * inv * w[7]);
+        if (FP8) {
+          float y[8];
+          unpack8e<E>(o, y);
+          store8(dy, off[k] / 2, quant4_fp8(y[0], y[1], y[2], y[3], scale_inv),
+                 quant4_fp8(y[4], y[5], y[6], y[7], scale_inv));
+        } else {
+          store16(dy, off[k], o);
+        }
       }
     }
     TW_STAMP(row, 4);          // y stores issued
     TW_STAMP_DRAINED(row, 5);  // every store of the row acknowledged
-  }
+    row += grid;
+    phase ^= 1;
+  } while (row < num_tokens);
 }
 
 template <int NP, int VPT, int MAXNT, bool HAS_RES, bool COPY, int Q>
 __global__ __launch_bounds__(MAXNT) void row_norm_bf16_kernel(
     PartialPtrs parts, int np_rt, void* y_out, void* residual, void* copy_out,
     const void* __restrict__ weight, const float* __restrict__ quant_scale,
-    float* __restrict__ row_scales, float eps, int num_tokens, int vec_per_row, float hidden) {
+    float* __restrict__ row_scales, float eps, int num_tokens, int vec_per_row, float hidden, int nt, int grid) {
   __shared__ float slots[2][kMaxChunks];
   __shared__ float max_slots[2][16];
   row_norm_vec_body<__bf16, NP, VPT, MAXNT, HAS_RES, COPY, Q>(parts, np_rt, y_out, residual, copy_out, weight,
                                                             quant_scale, row_scales, eps, num_tokens,
-                                                            vec_per_row, hidden, slots, max_slots);
+                                                            vec_per_row, hidden, nt, grid, slots, max_slots);
 }
 
 // fp16 tensors reach the library through the P = 1 ops only.
@@ -545,12 +552,12 @@ template <int VPT, int MAXNT, bool HAS_RES, bool COPY, int Q>
 __global__ __launch_bounds__(MAXNT) void row_norm_f16_kernel(
     PartialPtrs parts, void* y_out, void* residual, void* copy_out, const void* __restrict__ weight,
     const float* __restrict__ quant_scale, float* __restrict__ row_scales, float eps, int num_tokens,
-    int vec_per_row, float hidden) {
+    int vec_per_row, float hidden, int nt, int grid) {
   __shared__ float slots[2][kMaxChunks];
   __shared__ float max_slots[2][16];
   row_norm_vec_body<_Float16, 1, VPT, MAXNT, HAS_RES, COPY, Q>(parts, 1, y_out, residual, copy_out, weight,
                                                              quant_scale, row_scales, eps, num_tokens,
-                                                             vec_per_row, hidden, slots, max_slots);
+                                                             vec_per_row, hidden, nt, grid, slots, max_slots);
 }
 
 // ---------------------------------------------------------------------------
@@ -602,9 +609,9 @@ __device__ __forceinline__ void store16_device(__amdgpu_buffer_rsrc_t d, uint32_
 template <int NP, int VPT, bool XCD_ROWS>
 __global__ __launch_bounds__(1024) void row_norm_split_kernel(
     PartialPtrs parts, int np_rt, void* y_out, void* residual, const void* __restrict__ weight,
-    SplitRow* __restrict__ ws, float eps, int num_tokens, int vec_per_row, float hidden, int segs) {
+    SplitRow* __restrict__ ws, float eps, int num_tokens, int vec_per_row, float hidden, int segs, int nt) {
   __shared__ uint32_t arrivals_before;
-  const int nt = blockDim.x;
+  // nt = lanes per workgroup, as a kernel argument (see row_norm_vec_body)
   const int nwaves = nt >> 6;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int nchunks = (vec_per_row + 63) >> 6;
@@ -614,6 +621,10 @@ __global__ __launch_bounds__(1024) void row_norm_split_kernel(
   const int per_group = 8 * segs;
   const int row = XCD_ROWS ? (blockIdx.x / per_group) * 8 + (blockIdx.x & 7) : blockIdx.x / segs;
   const int seg = XCD_ROWS ? (blockIdx.x % per_group) >> 3 : blockIdx.x % segs;
+  // The first partial's pointer is demanded here so that its load goes out with the
+  // row count's: one round trip to the kernel arguments ahead of the test, and the loads
+  // that follow find their cache lines there.
+  asm volatile("" ::"s"(parts.p[0]));
   if (row >= num_tokens) return;
   const int chunk0 = seg * VPT * nwaves;  // first chunk of this segment
 
@@ -912,7 +923,7 @@ static int launch_vec(const RowNormArgs& a) {
 #define TW_LAUNCH_F16(VPT, MAXNT)                                                                \
   launch_kernel(row_norm_f16_kernel<VPT, MAXNT, HAS_RES, COPY, Q>, g, b, 0, a.stream,            \
                      a.parts, a.y, a.residual, a.copy_out, a.weight, a.quant_scale,              \
-                     a.row_scales, a.eps, (int)a.T, V, (float)a.H)
+                     a.row_scales, a.eps, (int)a.T, V, (float)a.H, sh.nt, a.grid)
     if (sh.vpt == 1) TW_LAUNCH_F16(1, 1024);
     else if (sh.vpt == 2) TW_LAUNCH_F16(2, 1024);
     else if (sh.maxnt == 256) TW_LAUNCH_F16(4, 256);
@@ -923,7 +934,7 @@ static int launch_vec(const RowNormArgs& a) {
 #define TW_LAUNCH(VPT, MAXNT)                                                                    \
   launch_kernel(row_norm_bf16_kernel<NP, VPT, MAXNT, HAS_RES, COPY, Q>, g, b, 0,                 \
                      a.stream, a.parts, a.np, a.y, a.residual, a.copy_out, a.weight,             \
-                     a.quant_scale, a.row_scales, a.eps, (int)a.T, V, (float)a.H)
+                     a.quant_scale, a.row_scales, a.eps, (int)a.T, V, (float)a.H, sh.nt, a.grid)
   if (sh.vpt == 1) TW_LAUNCH(1, 1024);
   else if (sh.vpt == 2) TW_LAUNCH(2, 1024);
   else if (sh.maxnt == 256) TW_LAUNCH(4, 256);
@@ -967,7 +978,7 @@ static void launch_split(const RowNormArgs& a, const SplitPlan& sp) {
   dim3 g((unsigned)(groups * 8 * sp.segs)), b((unsigned)(sp.nwaves * 64));
 #define TW_LAUNCH_SPLIT(VPT)                                                                     \
   launch_kernel(row_norm_split_kernel<NP, VPT, true>, g, b, 0, a.stream, a.parts, a.np, a.y,     \
-                a.residual, a.weight, a.split_ws, a.eps, (int)a.T, V, (float)a.H, sp.segs)
+                a.residual, a.weight, a.split_ws, a.eps, (int)a.T, V, (float)a.H, sp.segs, sp.nwaves * 64)
   if (sp.vpt == 1) TW_LAUNCH_SPLIT(1);
   else if (sp.vpt == 2) TW_LAUNCH_SPLIT(2);
   else TW_LAUNCH_SPLIT(4);

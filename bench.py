@@ -353,11 +353,12 @@ def time_ceilings(device):
     return out
 
 
-def time_timeline(cfg, device, launches=200):
-    """Runs the stamped build of the norm kernel `launches` times on rotating inputs and
-    reduces the per-row stamps (wall clock, 10 ns units) to a breakdown of one launch:
-    microseconds; `min`/`median`/`max` are over the rows of a launch, each then the
-    median over launches."""
+def time_timeline(cfg, device, launches=200, burst=6):
+    """Runs the stamped build of the norm kernel in `launches` bursts of `burst` back-to-back launches on
+    rotating inputs, keeps the stamps of each burst's last launch (a launch that starts on an idle GPU
+    begins 0.4 - 0.7 us later on half of the XCCs; one that follows another does not) and reduces the
+    per-row stamps (wall clock, 10 ns units) to a breakdown of one launch: microseconds;
+    `min`/`median`/`max` are over the rows of a launch, each then the median over launches."""
     import numpy as np
     import torch
     from tokenweave_amd import workloads as wl
@@ -370,23 +371,30 @@ def time_timeline(cfg, device, launches=200):
     for i in range(nsets):
         inp = wl.make_norm_inputs(cfg, device, seed_offset=i)
         sets.append((inp, (vp * cfg.P)(*[p.data_ptr() for p in inp.partials])))
+    slot = torch.zeros((cfg.T, 8), dtype=torch.int64, device=device)
     trace = torch.zeros((launches, cfg.T, 8), dtype=torch.int64, device=device)
 
-    def call(i, slot):
+    def call(i):
         inp, ptrs = sets[i % nsets]
         bench_check(L.twb_trace_reduce_add_rms_norm(ptrs, cfg.P, inp.partials[0].data_ptr(),
                                                     inp.residual.data_ptr(), inp.weight.data_ptr(), cfg.T, cfg.H,
-                                                    0, cfg.eps, trace[slot].data_ptr(), sp))
+                                                    0, cfg.eps, slot.data_ptr(), sp))
     for i in range(50):
-        call(i, 0)
+        call(i)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for i in range(launches):
-        call(50 + i, i)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    event_us = e0.elapsed_time(e1) * 1e3 / launches
+    n, event_ms = 50, []
+    for s in range(launches):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        call(n)
+        e0.record(stream)
+        for i in range(1, burst):
+            call(n + i)
+        e1.record(stream)
+        n += burst
+        torch.cuda.synchronize()
+        event_ms.append(e0.elapsed_time(e1) / (burst - 1))
+        trace[s].copy_(slot)
+    event_us = sorted(event_ms)[len(event_ms) // 2] * 1e3
     t = trace.cpu().numpy()
     st = t[:, :, :6].astype(np.float64) * 0.01          # 100 MHz wall clock -> us
     xcc = (t[:, :, 6] >> 32) & 0xf
@@ -399,14 +407,12 @@ def time_timeline(cfg, device, launches=200):
         return {"min": round(med(a.min(axis=1)), 2), "median": round(med(np.median(a, axis=1)), 2),
                 "max": round(med(a.max(axis=1)), 2)}
     span = rel[:, :, 5].max(axis=1)
-    gaps = st[1:, :, 0].min(axis=1) - st[:-1, :, 5].max(axis=1)
     out = {
-        "workload": cfg.name, "launches": launches,
+        "workload": cfg.name, "launches": launches, "burst": burst,
         "event_us_per_launch_with_stamps": round(event_us, 3),
         "first_row_begin_to_last_ack_us": {"median": round(med(span), 2), "min": round(float(span.min()), 2),
                                            "max": round(float(span.max()), 2)},
-        "last_ack_to_next_launch_first_row_us": {"median": round(med(gaps), 2), "min": round(float(gaps.min()), 2),
-                                                 "max": round(float(gaps.max()), 2)},
+        "launch_to_launch_minus_span_us": round(event_us - med(span), 2),
         "row_begin_after_first_row_us": rows_stat(rel[:, :, 0]),
         "loads_returned_after_row_begin_us": rows_stat(st[:, :, 1] - st[:, :, 0]),
         "loads_returned_after_first_row_us": rows_stat(rel[:, :, 1]),

@@ -30,59 +30,64 @@ struct Streams {
   const void* p[9];
 };
 
-// Per row: nine streams read with the norm kernel's loads.  WRITE: the folded value is
-// stored over the row in streams 0 and 8 (the norm's y and residual); otherwise nothing
-// is written unless the data matches a pattern that random inputs never produce.
-template <bool WRITE>
-__global__ __launch_bounds__(256) void stream_rows_kernel(Streams st, uint4* sink, int rows, int vec_per_row,
-                                                          int write_only) {
+// One workgroup per row (the launchers start exactly `rows` workgroups, so the kernels
+// neither test nor loop: like the norm kernel they make one round trip to their
+// arguments before the first load).
+// Per row: nine streams read with the norm kernel's loads.  MODE 0: read them (nothing is
+// written unless the data matches a pattern that random inputs never produce); 1: read
+// them and store the folded value over the row in streams 0 and 8 (the norm's y and
+// residual); 2: overwrite streams 0 and 8 and read nothing (what the memory system gives
+// the stores by themselves).
+template <int MODE>
+__global__ __launch_bounds__(256) void stream_rows_kernel(Streams st, uint4* sink, int vec_per_row) {
+  // all kernel arguments are demanded here, so that they are fetched in one round trip
+  asm volatile("" ::"s"(st.p[0]), "s"(st.p[1]), "s"(st.p[2]), "s"(st.p[3]), "s"(st.p[4]), "s"(st.p[5]),
+               "s"(st.p[6]), "s"(st.p[7]), "s"(st.p[8]), "s"(vec_per_row));
   const uint32_t row_bytes = (uint32_t)vec_per_row * 16u;
-  if (WRITE && write_only) {
-    // the two written streams alone: what the memory system gives the stores by themselves
-    for (int row = blockIdx.x; row < rows; row += gridDim.x) {
-      const __amdgpu_buffer_rsrc_t d0 = row_desc(st.p[0], row, row_bytes);
-      const __amdgpu_buffer_rsrc_t d8 = row_desc(st.p[8], row, row_bytes);
-      const uint4 v = make_uint4(row, threadIdx.x, 0x3f803f80u, 0x3f803f80u);
+  const int row = blockIdx.x;  // launched with one workgroup per row: no test, no loop
+  if (MODE == 2) {
+    const __amdgpu_buffer_rsrc_t d0 = row_desc(st.p[0], row, row_bytes);
+    const __amdgpu_buffer_rsrc_t d8 = row_desc(st.p[8], row, row_bytes);
+    const uint4 v = make_uint4(row, threadIdx.x, 0x3f803f80u, 0x3f803f80u);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) store16(d8, (threadIdx.x + k * 256) * 16u, v);
+    for (int k = 0; k < 4; ++k) store16(d8, (threadIdx.x + k * 256) * 16u, v);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) store16(d0, (threadIdx.x + k * 256) * 16u, v);
-    }
+    for (int k = 0; k < 4; ++k) store16(d0, (threadIdx.x + k * 256) * 16u, v);
     return;
   }
-  for (int row = blockIdx.x; row < rows; row += gridDim.x) {
-    uint4 a[4][9];
+  uint4 a[4][9];
 #pragma unroll
-    for (int s = 0; s < 9; ++s) {
-      const __amdgpu_buffer_rsrc_t d = row_desc(st.p[s], row, row_bytes);
+  for (int s = 0; s < 9; ++s) {
+    const __amdgpu_buffer_rsrc_t d = row_desc(st.p[s], row, row_bytes);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) a[k][s] = load16<kLoadStream>(d, (threadIdx.x + k * 256) * 16u);
+    for (int k = 0; k < 4; ++k) a[k][s] = load16<kLoadStream>(d, (threadIdx.x + k * 256) * 16u);
+  }
+  // every load of the row is in flight before the first use, as in the norm kernel
+  __builtin_amdgcn_sched_barrier(0);
+  uint4 f[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    f[k] = a[k][0];
+#pragma unroll
+    for (int s = 1; s < 9; ++s) {
+      f[k].x ^= a[k][s].x;
+      f[k].y ^= a[k][s].y;
+      f[k].z ^= a[k][s].z;
+      f[k].w ^= a[k][s].w;
     }
-    uint4 f[4];
+  }
+  if (MODE == 1) {
+    const __amdgpu_buffer_rsrc_t d0 = row_desc(st.p[0], row, row_bytes);
+    const __amdgpu_buffer_rsrc_t d8 = row_desc(st.p[8], row, row_bytes);
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      f[k] = a[k][0];
+    for (int k = 0; k < 4; ++k) store16(d8, (threadIdx.x + k * 256) * 16u, f[k]);
 #pragma unroll
-      for (int s = 1; s < 9; ++s) {
-        f[k].x ^= a[k][s].x;
-        f[k].y ^= a[k][s].y;
-        f[k].z ^= a[k][s].z;
-        f[k].w ^= a[k][s].w;
-      }
-    }
-    if (WRITE) {
-      const __amdgpu_buffer_rsrc_t d0 = row_desc(st.p[0], row, row_bytes);
-      const __amdgpu_buffer_rsrc_t d8 = row_desc(st.p[8], row, row_bytes);
+    for (int k = 0; k < 4; ++k) store16(d0, (threadIdx.x + k * 256) * 16u, f[k]);
+  } else {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) store16(d8, (threadIdx.x + k * 256) * 16u, f[k]);
-#pragma unroll
-      for (int k = 0; k < 4; ++k) store16(d0, (threadIdx.x + k * 256) * 16u, f[k]);
-    } else {
-#pragma unroll
-      for (int k = 0; k < 4; ++k)
-        if (f[k].x == 0x5eed5eedu && f[k].y == 0x0badf00du && f[k].z == 0x12345678u && f[k].w == 0x9abcdef0u)
-          sink[threadIdx.x] = f[k];
-    }
+    for (int k = 0; k < 4; ++k)
+      if (f[k].x == 0x5eed5eedu && f[k].y == 0x0badf00du && f[k].z == 0x12345678u && f[k].w == 0x9abcdef0u)
+        sink[threadIdx.x] = f[k];
   }
 }
 
@@ -97,7 +102,8 @@ __device__ __forceinline__ void wait_loads_outstanding() {
 __global__ __launch_bounds__(256) void stream_rows_trace_kernel(Streams st, unsigned long long* trace, int rows,
                                                                 int vec_per_row) {
   const uint32_t row_bytes = (uint32_t)vec_per_row * 16u;
-  for (int row = blockIdx.x; row < rows; row += gridDim.x) {
+  {
+    const int row = blockIdx.x;  // launched with one workgroup per row: no test, no loop
     unsigned long long* t = trace + (size_t)row * 16;
     const bool rec = threadIdx.x == 0;
     if (rec) t[0] = wall_clock64();
@@ -317,12 +323,11 @@ TW_API int twb_stream_rows(const void* const* streams, void* sink, int64_t rows,
   }
   const dim3 g((unsigned)rows), b(256);
   hipStream_t hs = static_cast<hipStream_t>(stream);
-  if (write)
-    tw::launch_kernel(twb::stream_rows_kernel<true>, g, b, 0, hs, st, static_cast<uint4*>(sink), (int)rows,
-                      (int)(hidden_size / 8), write == 2 ? 1 : 0);
-  else
-    tw::launch_kernel(twb::stream_rows_kernel<false>, g, b, 0, hs, st, static_cast<uint4*>(sink), (int)rows,
-                      (int)(hidden_size / 8), 0);
+  uint4* sk = static_cast<uint4*>(sink);
+  const int vec = (int)(hidden_size / 8);
+  if (write == 2) tw::launch_kernel(twb::stream_rows_kernel<2>, g, b, 0, hs, st, sk, vec);
+  else if (write) tw::launch_kernel(twb::stream_rows_kernel<1>, g, b, 0, hs, st, sk, vec);
+  else tw::launch_kernel(twb::stream_rows_kernel<0>, g, b, 0, hs, st, sk, vec);
   return tw::finish_launch("stream_rows");
 }
 
@@ -354,15 +359,21 @@ TW_API int twb_empty(int grid, int block, void* stream) {
 // tw_reduce_add_rms_norm with timeline stamps: trace is num_tokens x 8 uint64 of device
 // memory.  Per row: [0] row begins, [1] all loads returned, [2] residual stores issued,
 // [3] row sum known, [4] y stores issued, [5] all stores acknowledged (wall clock, 10 ns
-// units), [6] XCC id << 32 | HW_ID, [7] unused.  Synchronous on entry (it sets a device
-// global), asynchronous afterwards.
+// units), [6] XCC id << 32 | HW_ID, [7] unused.  The first call with a given trace buffer
+// is synchronous on entry (it sets a device global); further calls with the same buffer
+// are asynchronous, so a burst of launches runs back to back and leaves the stamps of its
+// last launch.
 TW_API int twb_trace_reduce_add_rms_norm(const void* const* partials, int num_partials, void* y, void* residual,
                                          const void* weight, int64_t num_tokens, int64_t hidden_size,
                                          int max_ctas, float epsilon, void* trace, void* stream) {
   if (!trace) return tw::set_error(TW_ERR_INVALID_ARGUMENT, "trace: null trace buffer");
   unsigned long long* buf = static_cast<unsigned long long*>(trace);
-  if (hipMemcpyToSymbol(HIP_SYMBOL(tw::g_trace), &buf, sizeof(buf)) != hipSuccess)
-    return tw::set_error(TW_ERR_LAUNCH, "trace: could not set the trace pointer");
+  static unsigned long long* current = nullptr;  // bench.py calls from one thread, on one device
+  if (buf != current) {
+    if (hipMemcpyToSymbol(HIP_SYMBOL(tw::g_trace), &buf, sizeof(buf)) != hipSuccess)
+      return tw::set_error(TW_ERR_LAUNCH, "trace: could not set the trace pointer");
+    current = buf;
+  }
   return tw::run_row_norm("trace_reduce_add_rms_norm", partials, num_partials, y, residual, nullptr, weight,
                           nullptr, num_tokens, hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true, stream);
 }

@@ -55,26 +55,31 @@ struct PartialPtrs {
 #ifdef TW_TRACE
 __device__ unsigned long long* g_trace;
 constexpr int kTraceSlots = 8;
-#define TW_STAMP(row, i)                                                                         \
-  do {                                                                                           \
-    if (threadIdx.x == 0) g_trace[(size_t)(row) * kTraceSlots + (i)] = wall_clock64();           \
-  } while (0)
+// The stamps of a row are collected in registers and written out after its last one, so
+// that neither the trace pointer's load nor the stamp stores sit in the row's way.
+#define TW_STAMP_BEGIN unsigned long long tw_stamps[kTraceSlots] = {}
+#define TW_STAMP(row, i) tw_stamps[i] = wall_clock64()
 #define TW_STAMP_DRAINED(row, i)                                                                 \
   do {                                                                                           \
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                             \
     TW_STAMP(row, i);                                                                            \
   } while (0)
 #define TW_STAMP_HWID(row, i)                                                                    \
+  tw_stamps[i] = ((unsigned long long)__builtin_amdgcn_s_getreg((4 - 1) << 11 | 20) << 32) |     \
+                 (unsigned)__builtin_amdgcn_s_getreg((32 - 1) << 11 | 4)
+#define TW_STAMP_END(row)                                                                        \
   do {                                                                                           \
-    if (threadIdx.x == 0)                                                                        \
-      g_trace[(size_t)(row) * kTraceSlots + (i)] =                                               \
-          ((unsigned long long)__builtin_amdgcn_s_getreg((4 - 1) << 11 | 20) << 32) |            \
-          (unsigned)__builtin_amdgcn_s_getreg((32 - 1) << 11 | 4);                               \
+    if (threadIdx.x == 0) {                                                                      \
+      for (int tw_i = 0; tw_i < kTraceSlots; ++tw_i)                                             \
+        g_trace[(size_t)(row) * kTraceSlots + tw_i] = tw_stamps[tw_i];                           \
+    }                                                                                            \
   } while (0)
 #else
+#define TW_STAMP_BEGIN
 #define TW_STAMP(row, i)
 #define TW_STAMP_DRAINED(row, i)
 #define TW_STAMP_HWID(row, i)
+#define TW_STAMP_END(row)
 #endif
 
 // ---------------------------------------------------------------------------
@@ -372,6 +377,7 @@ __device__ __forceinline__ void row_norm_vec_body(
     float s[VPT][8];
     uint4 first[VPT];
     uint4 wv[VPT];     // the weight row is fetched per token row, behind the row's own loads
+    TW_STAMP_BEGIN;
     TW_STAMP(row, 0);  // row begins
     TW_STAMP_HWID(row, 6);
     const __amdgpu_buffer_rsrc_t dr = row_desc(HAS_RES ? residual : parts.p[0], row, row_bytes);
@@ -530,6 +536,7 @@ __device__ __forceinline__ void row_norm_vec_body(
     }
     TW_STAMP(row, 4);          // y stores issued
     TW_STAMP_DRAINED(row, 5);  // every store of the row acknowledged
+    TW_STAMP_END(row);
     row += grid;
     phase ^= 1;
   } while (row < num_tokens);

@@ -45,7 +45,7 @@ ROTATION_BYTES = 4 << 30      # distinct operand bytes cycled through before any
 # kernel of known size), transcribed from the summary named beside each figure; this run
 # does not measure them.  Workloads without a counter run: None.
 MEASURED_TRAFFIC_BYTES = {
-    "c2_llama70b_tp8_shard@T256": (46366607, "profiles/row_norm_bf16_c2_T256_pmc_traffic.md"),
+    "c2_llama70b_tp8_shard@T256": (46375250, "profiles/row_norm_bf16_c2_T256_pmc_traffic.md"),
 }
 # dominant kernel of a workload, as rocprofv3 names it
 KERNEL_NAMES = {"c2_llama70b_tp8_shard@T256": "row_norm_bf16_kernel<8,4,256,true,false,0>"}

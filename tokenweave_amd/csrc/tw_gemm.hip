@@ -44,6 +44,7 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int LDS_ROW = BK + 8;  // elements; 144-byte row pitch
@@ -431,8 +432,12 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
           // 8-byte LDS reads: the padded row pitch keeps rows 8-byte, not 16-byte, aligned
           const uint2 lo = *reinterpret_cast<const uint2*>(patch + row * PATCH_ROW + rd_chunk * 16);
           const uint2 hi = *reinterpret_cast<const uint2*>(patch + row * PATCH_ROW + rd_chunk * 16 + 8);
-          if (rd_lane && r + rd_row < 32 && m < M && n < N)
-            *reinterpret_cast<uint4*>(out + (size_t)m * ldc + n) = make_uint4(lo.x, lo.y, hi.x, hi.y);
+          // streaming stores: the tile is not read again by this kernel, and whoever reads
+          // it next (the norm kernel) runs on other XCDs; 1 - 3.5 % faster than default stores
+          if (rd_lane && r + rd_row < 32 && m < M && n < N) {
+            const u32x4_t v = {lo.x, lo.y, hi.x, hi.y};
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(out + (size_t)m * ldc + n));
+          }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();

@@ -881,7 +881,10 @@ static int default_grid(int64_t num_tokens) {
 //   * T >= 224: four vectors per lane in workgroups of at most 256 lanes, every
 //     load of the row in flight at once (fastest from 256 to 8192 rows); the P = 1
 //     ops, half of whose traffic is stores, run 0.3 - 2.5 % faster with two vectors
-//     per lane from 1024 rows on (512 lanes at hidden size 8192);
+//     per lane from 1024 rows on (512 lanes at hidden size 8192); rows between 512
+//     and 1024 vectors, whose quarter does not fill a 256-lane workgroup, do so from
+//     8192 rows on (hidden size 6144: 2.5 - 2.9 % faster at 8192 and 16384 rows, 5 %
+//     slower at 1024 and 2048; hidden size 8192 is 2 - 6 % slower that way at any size);
 //   * rows longer than 1024 vectors: two vectors per lane up to 2048 vectors, four
 //     up to 4096 (one partial at a time).  Longer rows take the element-wise kernel.
 struct VecShape { int vpt, nt, maxnt; };
@@ -892,6 +895,7 @@ static bool vec_shape(int V, int64_t T, int np, VecShape* sh) {
     if (T < 48 || V < 128) vpt = 1;
     else if (T < 224 || V < 256) vpt = 2;
     else if (np == 1 && T >= 1024 && V >= 512) vpt = 2;
+    else if (T >= 8192 && V > 512 && V < 1024) vpt = 2;
     else { vpt = 4; maxnt = 256; }
   } else if (V <= 2048) vpt = 2;
   else if (V <= 4096) vpt = 4;

@@ -59,31 +59,32 @@ _BENCH_LIB = None
 
 
 def bench_lib():
-    """tokenweave_amd/libtw_bench.so: measurement-only kernels (plain copy, row streams, empty
+    """benchlib/libtw_bench.so: measurement-only kernels (plain copy, row streams, empty
     kernel) and the norm kernels compiled with timeline stamps.  Built by `make -C
-    tokenweave_amd/csrc`; the product never loads it."""
+    benchlib`; the package neither builds nor loads it."""
     global _BENCH_LIB
     if _BENCH_LIB is None:
-        path = os.path.join(ROOT, "tokenweave_amd", "libtw_bench.so")
+        path = os.path.join(ROOT, "benchlib", "libtw_bench.so")
         if not os.path.exists(path):
-            sys.exit(f"{path} is missing: build it with `make -C tokenweave_amd/csrc`")
+            sys.exit(f"{path} is missing: build it with `make -C benchlib`")
         L = ctypes.CDLL(path)
         vp, i64, ci, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
         L.twb_copy_bytes.argtypes = [vp, vp, i64, vp]
         L.twb_stream_rows.argtypes = [ctypes.POINTER(vp), vp, i64, i64, ci, vp]
         L.twb_trace_stream_rows.argtypes = [ctypes.POINTER(vp), vp, i64, i64, vp]
         L.twb_empty.argtypes = [ci, ci, vp]
+        L.twb_clock_probe.argtypes = [vp, ci, vp]
         L.twb_trace_reduce_add_rms_norm.argtypes = [ctypes.POINTER(vp), ci, vp, vp, vp, i64, i64, ci, f32, vp, vp]
         L.twb_gemm_loop.argtypes = [ci, ci, i64, vp, vp, vp, ci, vp]
         L.twb_lds_read_rate.argtypes = [ci, ci, ci, vp, vp, vp, ci, vp]
-        L.tw_last_error.restype = ctypes.c_char_p
+        L.twb_last_error.restype = ctypes.c_char_p
         _BENCH_LIB = L
     return _BENCH_LIB
 
 
 def bench_check(rc):
     if rc:
-        raise RuntimeError(bench_lib().tw_last_error().decode())
+        raise RuntimeError(bench_lib().twb_last_error().decode())
 
 
 def parse_args():
@@ -394,6 +395,7 @@ def time_timeline(cfg, device, launches=200, burst=6):
         torch.cuda.synchronize()
         event_ms.append(e0.elapsed_time(e1) / (burst - 1))
         trace[s].copy_(slot)
+    bench_check(L.twb_trace_end())   # later launches write no stamps: `slot` may be freed
     event_us = sorted(event_ms)[len(event_ms) // 2] * 1e3
     t = trace.cpu().numpy()
     st = t[:, :, :6].astype(np.float64) * 0.01          # 100 MHz wall clock -> us
@@ -537,15 +539,45 @@ def time_norm_warm(cfg, steps, max_ctas, device):
     return e0.elapsed_time(e1) * 1e3 / steps
 
 
+def host_cpu():
+    """(model string, physical cores, logical CPUs) of the host, from /proc/cpuinfo."""
+    model, cores, logical = "unknown", set(), 0
+    try:
+        phys = core = None
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                key, _, val = line.partition(":")
+                key, val = key.strip(), val.strip()
+                if key == "model name":
+                    model = val
+                elif key == "processor":
+                    logical += 1
+                elif key == "physical id":
+                    phys = val
+                elif key == "core id":
+                    core = val
+                elif not key and phys is not None and core is not None:
+                    cores.add((phys, core))
+                    phys = core = None
+        if phys is not None and core is not None:
+            cores.add((phys, core))
+    except OSError:
+        pass
+    return model, len(cores) or None, logical or (os.cpu_count() or 1)
+
+
 def cpu_baseline(cfg, budget_s):
     """Times the CPU checker on a bounded sample of the workload: the same shapes (rows
     capped at 1024), rotating through input sets of 1 GiB in total so that, like the GPU
-    legs, every call reads memory and not a cache, repeated for `budget_s` seconds."""
+    legs, every call reads memory and not a cache.  Two legs: OpenMP over rows with all the
+    threads this process is given (OMP_NUM_THREADS, else the logical CPUs) for two thirds of
+    `budget_s` seconds -> value, cores; and one thread for the rest -> single_thread."""
     import numpy as np
     import torch
     from oracle import tw_oracle as O
     from tokenweave_amd import workloads as wl
-    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    model, physical, logical = host_cpu()
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or logical
     rows = min(cfg.T, 1024)
     sample = cfg.with_tokens(rows)
     bits = lambda t: np.ascontiguousarray(t.contiguous().view(torch.int16).numpy().view(np.uint16))
@@ -555,49 +587,65 @@ def cpu_baseline(cfg, budget_s):
         inp = wl.make_norm_inputs(sample, "cpu", seed_offset=i)
         r = bits(inp.residual)
         sets.append(([bits(p) for p in inp.partials], r, bits(inp.weight), np.empty_like(r)))
-    for parts, r, w, y in sets[:2]:   # warm-up (page faults, thread pool)
-        O.reduce_add_rms_norm(parts, r, w, cfg.eps, y=y)
-    times, t_end = [], time.perf_counter() + budget_s
-    while len(times) < 3 or time.perf_counter() < t_end:
-        parts, r, w, y = sets[len(times) % nsets]
-        t0 = time.perf_counter()
-        O.reduce_add_rms_norm(parts, r, w, cfg.eps, y=y)
-        times.append(time.perf_counter() - t0)
-    med = statistics.median(times)
+    O.lib()
+    gomp = ctypes.CDLL("libgomp.so.1")   # the OpenMP runtime the checker is linked against
+
+    def leg(nthreads, seconds):
+        gomp.omp_set_num_threads(nthreads)
+        for parts, r, w, y in sets[:2]:   # warm-up (page faults, thread pool)
+            O.reduce_add_rms_norm(parts, r, w, cfg.eps, y=y)
+        times, t_end = [], time.perf_counter() + seconds
+        while len(times) < 3 or time.perf_counter() < t_end:
+            parts, r, w, y = sets[len(times) % nsets]
+            t0 = time.perf_counter()
+            O.reduce_add_rms_norm(parts, r, w, cfg.eps, y=y)
+            times.append(time.perf_counter() - t0)
+        return statistics.median(times), len(times)
+
+    med, n = leg(threads, budget_s * 2.0 / 3.0)
+    med1, n1 = leg(1, budget_s / 3.0)
+    gomp.omp_set_num_threads(threads)
     return {"value": round(sample.bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads,
-            "kind": "port",
-            "sample": f"{len(times)} calls in {budget_s:.0f} s of P={sample.P} T={rows} H={sample.H} "
+            "kind": "port", "cpu_model": model, "physical_cores": physical, "logical_cpus": logical,
+            "single_thread": {"value": round(sample.bytes / med1 / 1e9, 3), "unit": "GB/s", "cores": 1,
+                              "us_per_call": round(med1 * 1e6, 1), "calls": n1},
+            "sample": f"{n} calls in {budget_s * 2 / 3:.0f} s of P={sample.P} T={rows} H={sample.H} "
                       f"({sample.bytes} algorithmic bytes each) over {nsets} rotating input sets, "
-                      f"median {med * 1e6:.0f} us/call, OpenMP over rows with {threads} threads"}
-
-
-_WEAVE_STREAMS = None
+                      f"median {med * 1e6:.0f} us/call, OpenMP over rows with {threads} threads; then "
+                      f"{n1} calls in {budget_s / 3:.0f} s with one thread, median {med1 * 1e6:.0f} us/call"}
 
 
 def weave_streams():
-    """The two streams of every weave measurement, created once: HIP spreads streams over a
-    few hardware queues (4 by default) in creation order, and two streams that land on one
-    queue run their kernels one after the other."""
-    global _WEAVE_STREAMS
-    if _WEAVE_STREAMS is None:
-        import torch
-        _WEAVE_STREAMS = (torch.cuda.Stream(), torch.cuda.Stream())
-    return _WEAVE_STREAMS
+    """The two streams of every weave measurement, created once (the tuner's pair: HIP spreads
+    streams over a few hardware queues, 4 by default, in creation order, and two streams that
+    land on one queue run their kernels one after the other)."""
+    from tokenweave_amd.tune_weave import weave_streams as pair
+    return pair()
 
 
-def time_weave(device, form="eight_partials", gemm_caps=(128,), norm_cap=0, steps=200):
+WEAVE_REGIONS = 11   # rounds in which the legs of a weave measurement take turns
+
+
+def time_weave(device, form="eight_partials", gemm_caps=(128,), norm_cap=0, steps=20, regions=WEAVE_REGIONS):
     """Config 5: the bf16 MFMA GEMM of the 2458-row split on the current stream overlapped with
     the fused norm of the 1638-row split on a second stream.  form "eight_partials": the
     producer of all P = 8 row-parallel partial sums of the split (one launch,
     tw_gemm_bf16_nt_partials, into the 8 staging slots); "one_partial": one rank's GEMM.
-    Every figure is the mean over `steps` back-to-back stages bracketed by HIP events; the
-    norm inputs rotate through 8 sets (2.4 GB) so it reads cold HBM, the GEMM outputs through
-    as many staging buffers.  Calls are pre-bound (arguments validated once by the public
-    shims) so that the host enqueues a stage faster than the GPU runs it.  The overlapped
-    stage is timed for every GEMM compute-unit budget in `gemm_caps`; the best is reported."""
+
+    The legs — GEMM alone, norm alone, both on one stream (serial), and the two-stream stage
+    for every GEMM compute-unit budget in `gemm_caps` — take turns region by region
+    (`regions` rounds; in each, every leg runs 2 untimed and `steps` timed stages between
+    HIP events), and each figure is the median over the rounds: every leg sees the same
+    mix of clock and power states, where back-to-back legs of seconds each would not.  A
+    one-wave clock probe follows each leg's timed stages and reads the shader clock the
+    leg left behind.  The serial leg is also timed with an event between its two kernels
+    (`*_us_in_serial`).  The norm inputs rotate through 8 sets (2.4 GB) so it reads cold HBM, the GEMM
+    outputs through as many staging buffers.  Calls are pre-bound (arguments validated once
+    by the public shims) so that the host enqueues a stage faster than the GPU runs it."""
     import torch
     from tokenweave_amd import _custom_ops as ops
     from tokenweave_amd import workloads as wl
+    from tokenweave_amd.tune_weave import interleaved_medians
     cfg = wl.C5_NORM
     P = 8 if form == "eight_partials" else 1
     R = 4 if P == 8 else 8
@@ -633,34 +681,66 @@ def time_weave(device, form="eight_partials", gemm_caps=(128,), norm_cap=0, step
             main_s.wait_stream(side_s)
         return stage
 
-    def timed(step):
-        torch.cuda.synchronize()
-        with torch.cuda.stream(main_s):
-            for i in range(5):
-                step(i)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(main_s)
-            for i in range(steps):
-                step(i)
-            e1.record(main_s)
-            torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / steps
+    legs = {"gemm": lambda i: gemm(i, 0, main_s), "norm": lambda i: norm(i, 0, main_s),
+            "serial": lambda i: (gemm(i, 0, main_s), norm(i, 0, main_s))}
+    for cap in gemm_caps:
+        legs[f"weave/{cap}"] = weave(cap)
 
-    t_a = timed(lambda i: gemm(i, 0, main_s))
-    t_b = timed(lambda i: norm(i, 0, main_s))
-    t_ser = timed(lambda i: (gemm(i, 0, main_s), norm(i, 0, main_s)))
-    by_cap = {cap: timed(weave(cap)) for cap in gemm_caps}
+    # shader clock right after each leg's timed stages
+    BL = bench_lib()
+    probe_out = torch.zeros((len(legs) * regions, 2), dtype=torch.int64, device=device)
+    probes = {name: [] for name in legs}
+
+    def probe(name):
+        k = sum(len(v) for v in probes.values())
+        bench_check(BL.twb_clock_probe(probe_out[k].data_ptr(), 20, main_s.cuda_stream))
+        probes[name].append(k)
+
+    res = interleaved_medians(legs, main_s, steps, regions=regions, after_region=probe)
+    pr = probe_out.cpu().numpy().astype(float)
+    clock = {name: round(statistics.median(pr[k, 0] / max(pr[k, 1], 1.0) / 10.0 for k in ks), 3)
+             for name, ks in probes.items()}   # cycles per 10 ns tick -> GHz
+
+    # the serial stage with an event between its kernels: what each takes inside the serial stage
+    g_in, n_in = [], []
+    with torch.cuda.stream(main_s):
+        it = 0
+        for _ in range(regions):
+            evs = []
+            for _ in range(steps):
+                e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+                e[0].record(main_s)
+                gemm(it, 0, main_s)
+                e[1].record(main_s)
+                norm(it, 0, main_s)
+                e[2].record(main_s)
+                evs.append(e)
+                it += 1
+            torch.cuda.synchronize()
+            g_in.append(statistics.mean(e[0].elapsed_time(e[1]) for e in evs[2:]) * 1e3)
+            n_in.append(statistics.mean(e[1].elapsed_time(e[2]) for e in evs[2:]) * 1e3)
+
+    t_a, t_b, t_ser = res["gemm"]["us"], res["norm"]["us"], res["serial"]["us"]
+    by_cap = {cap: res[f"weave/{cap}"]["us"] for cap in gemm_caps}
     best_cap = min(by_cap, key=by_cap.get)
     t_ovl = by_cap[best_cap]
     flops = 2.0 * P * Ta * N * K
+    # serial is two kernels that cannot overlap: it cannot undercut the longer one, and it
+    # should be the sum of the two alone up to what the different duty cycle does to the clock
+    consistent = t_ser >= max(t_a, t_b) * 0.995 and abs(t_ser - (t_a + t_b)) <= 0.05 * (t_a + t_b)
     out = {"form": form, "gemm_us": t_a, "norm_us": t_b, "serial_us": t_ser, "overlap_us": t_ovl,
-           "speedup": t_ser / t_ovl, "overlap_eff": (t_ser - t_ovl) / min(t_a, t_b),
+           "speedup": t_ser / t_ovl,
+           "overlap_eff": (t_ser - t_ovl) / min(t_a, t_b) if consistent else None,
+           "legs_consistent": consistent,
+           "serial_vs_sum_of_alone": t_ser / (t_a + t_b),
+           "gemm_us_in_serial": statistics.median(g_in), "norm_us_in_serial": statistics.median(n_in),
+           "us_min_max": {k: [round(v["min"], 2), round(v["max"], 2)] for k, v in res.items()},
+           "shader_clock_ghz_after_leg": clock,
            "gemm_tflops_alone": flops / t_a / 1e6,
            "gemm_mfma_util_alone": flops / t_a / 1e6 / MFMA_BF16_PEAK_TFLOPS,
            "gemm_mfma_util_in_stage": flops / t_ovl / 1e6 / MFMA_BF16_PEAK_TFLOPS,
            "norm_gbps_alone": cfg.bytes / t_b / 1e3, "norm_gbps_in_stage": cfg.bytes / t_ovl / 1e3,
-           "norm_cap": norm_cap, "gemm_cus": best_cap, "stages_timed": steps,
+           "norm_cap": norm_cap, "gemm_cus": best_cap, "stages_per_region": steps, "regions": regions,
            "overlap_us_by_gemm_cus": {str(c): round(v, 2) for c, v in by_cap.items()}}
     del gemms, norms, stages, inps, gs
     torch.cuda.empty_cache()
@@ -758,8 +838,10 @@ def weave_block(device, steps):
                         "the 1638-row split, H=8192",
             "definitions": "serial = both kernels on one stream; overlap = GEMM capped to gemm_cus compute "
                            "units on the current stream, norm on a second stream; speedup = serial/overlap; "
-                           "overlap_eff = (serial - overlap)/min(gemm, norm); MFMA utilisation against "
-                           "2.5 PFLOP/s dense bf16",
+                           "overlap_eff = (serial - overlap)/min(gemm, norm), null unless serial >= max(gemm, "
+                           "norm) and |serial - (gemm + norm)| <= 5 %; every leg is the median of "
+                           "`regions` interleaved regions of `stages_per_region` stages; MFMA utilisation "
+                           "against 2.5 PFLOP/s dense bf16",
             "eight_partials": time_weave(device, "eight_partials", caps, steps=steps),
             "one_partial": time_weave(device, "one_partial", caps, steps=steps)}
 
@@ -796,7 +878,7 @@ def main():
         print(json.dumps({"gemm_limits": time_gemm_limits(device)}), flush=True)
         return
     if args.weave_only:
-        print(json.dumps({"weave": weave_block(device, min(args.steps, 200))}), flush=True)
+        print(json.dumps({"weave": weave_block(device, 20)}), flush=True)
         return
     log(f"[bench] {torch.cuda.get_device_name(0)}; workload {cfg.name}: P={cfg.P} T={cfg.T} "
         f"H={cfg.H} bytes/call={cfg.bytes}")
@@ -834,7 +916,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
         log(f"[bench] cpu_baseline {out['cpu_baseline']}")
     if not args.no_weave:
-        out["weave"] = weave_block(device, 100)
+        out["weave"] = weave_block(device, 20)
         log(f"[bench] weave {out['weave']}")
     if args.calibration_copy:
         calibration_copies(device)

@@ -1,5 +1,7 @@
-// libtw_bench.so — kernels that exist for MEASUREMENT only; bench.py loads this
-// library, the product (libtokenweave_amd.so and the Python package) never does.
+// libtw_bench.so — kernels that exist for MEASUREMENT and TESTING only; bench.py and the
+// tests load this library, the product (libtokenweave_amd.so and the Python package)
+// never does.  The library's own sources are compiled into it, but none of the tw_*
+// entry points is exported from here: only the twb_* functions below are.
 //
 //  * the library's own norm kernels compiled with timeline stamps (TW_TRACE): the
 //    same source, plus per-row wall-clock stamps written to a caller's buffer;
@@ -13,13 +15,21 @@
 //  * the main loop of the big GEMM kernel put together from its parts (MFMAs, fragment
 //    reads from LDS, operand slabs global -> LDS, the barrier per k-slab) on operands that
 //    stay in the L2s, and the rate at which waves get 16-byte LDS reads through: what the
-//    loop itself can reach on this machine, apart from tile prologue and epilogue.
+//    loop itself can reach on this machine, apart from tile prologue and epilogue;
+//  * the split-row kernel WITHOUT its row-to-XCD placement (the segments of a row spread
+//    over the XCDs), which the product never launches: the tests run it against the same
+//    bits to pin that the cross-workgroup hand-over does not depend on the placement.
 #define TW_TRACE 1
+#define TW_API __attribute__((visibility("hidden")))
+#define TWB_API __attribute__((visibility("default")))
 #include "tw_api.hip"
 #include "tw_gemm.hip"
 #include "tw_norm.hip"
 
 namespace twb {
+
+// host copy of the device-side trace pointer (tw::g_trace): null outside a traced burst
+static unsigned long long* g_trace_current = nullptr;
 
 using tw::kLoadStream;
 using tw::load16;
@@ -149,6 +159,22 @@ __global__ __launch_bounds__(256) void copy16_kernel(uint4* __restrict__ dst, co
 }
 
 __global__ void empty_kernel() {}
+
+// One wave that watches both clocks for `ticks` units of the constant-rate wall clock
+// (10 ns each): out[0] = shader-clock cycles, out[1] = wall-clock ticks that went by.  The
+// ratio is the shader clock the compute unit ran at during the window.
+__global__ __launch_bounds__(64) void clock_probe_kernel(long long* out, long long ticks) {
+  const long long t0 = wall_clock64();
+  const long long c0 = __builtin_readcyclecounter();
+  long long t1 = t0;
+  // bounded: the wall clock advances whatever else happens, so the wave always leaves
+  while (t1 - t0 < ticks) t1 = wall_clock64();
+  const long long c1 = __builtin_readcyclecounter();
+  if (threadIdx.x == 0) {
+    out[0] = c1 - c0;
+    out[1] = t1 - t0;
+  }
+}
 
 
 // The k loop of gemm_bf16_nt_big_kernel<5, 2> (eight waves, 160 x 64 wave tiles, 320 x 256 x 64
@@ -291,7 +317,7 @@ __global__ __launch_bounds__(1024) void lds_read_rate_kernel(int iters, int dma,
 extern "C" {
 
 // dst[0, nbytes) <- src[0, nbytes): grid-stride copy, 16 bytes per lane, default cache policy.
-TW_API int twb_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
+TWB_API int twb_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
   if (nbytes < 0 || nbytes % 16 != 0 || !dst || !src ||
       ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u))
     return tw::set_error(TW_ERR_INVALID_ARGUMENT, "copy: needs 16-byte aligned pointers and size");
@@ -310,7 +336,7 @@ TW_API int twb_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stre
 // at most: hidden_size <= 8192, hidden_size % 8 == 0).  write = 0: read the nine streams;
 // 1: read them and overwrite streams 0 and 8; 2: overwrite streams 0 and 8, read nothing.
 // sink: 4 KiB of device memory (never written with random data).
-TW_API int twb_stream_rows(const void* const* streams, void* sink, int64_t rows, int64_t hidden_size,
+TWB_API int twb_stream_rows(const void* const* streams, void* sink, int64_t rows, int64_t hidden_size,
                            int write, void* stream) {
   if (!streams || !sink || rows < 1 || rows > INT32_MAX || hidden_size < 8 || hidden_size > 8192 ||
       hidden_size % 8 != 0)
@@ -332,7 +358,7 @@ TW_API int twb_stream_rows(const void* const* streams, void* sink, int64_t rows,
 }
 
 // twb_stream_rows(write = 1) with arrival stamps; trace: rows x 16 uint64 of device memory.
-TW_API int twb_trace_stream_rows(const void* const* streams, void* trace, int64_t rows, int64_t hidden_size,
+TWB_API int twb_trace_stream_rows(const void* const* streams, void* trace, int64_t rows, int64_t hidden_size,
                                  void* stream) {
   if (!streams || !trace || rows < 1 || rows > INT32_MAX || hidden_size < 8 || hidden_size > 8192 ||
       hidden_size % 8 != 0)
@@ -349,11 +375,21 @@ TW_API int twb_trace_stream_rows(const void* const* streams, void* trace, int64_
   return tw::finish_launch("trace_stream_rows");
 }
 
-TW_API int twb_empty(int grid, int block, void* stream) {
+TWB_API int twb_empty(int grid, int block, void* stream) {
   if (grid < 1 || block < 1 || block > 1024) return tw::set_error(TW_ERR_INVALID_ARGUMENT, "empty: bad launch shape");
   tw::launch_kernel(twb::empty_kernel, dim3((unsigned)grid), dim3((unsigned)block), 0,
                     static_cast<hipStream_t>(stream));
   return tw::finish_launch("empty");
+}
+
+// Shader clock over a window of `microseconds` (1 .. 1000) on one compute unit: out is two
+// int64 of device memory, {shader cycles, 10 ns wall-clock ticks}.
+TWB_API int twb_clock_probe(void* out, int microseconds, void* stream) {
+  if (!out || microseconds < 1 || microseconds > 1000)
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "clock_probe: bad argument");
+  tw::launch_kernel(twb::clock_probe_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                    static_cast<long long*>(out), (long long)microseconds * 100);
+  return tw::finish_launch("clock_probe");
 }
 
 // tw_reduce_add_rms_norm with timeline stamps: trace is num_tokens x 8 uint64 of device
@@ -362,22 +398,80 @@ TW_API int twb_empty(int grid, int block, void* stream) {
 // units), [6] XCC id << 32 | HW_ID, [7] unused.  The first call with a given trace buffer
 // is synchronous on entry (it sets a device global); further calls with the same buffer
 // are asynchronous, so a burst of launches runs back to back and leaves the stamps of its
-// last launch.
-TW_API int twb_trace_reduce_add_rms_norm(const void* const* partials, int num_partials, void* y, void* residual,
+// last launch.  Call twb_trace_end() before the trace buffer is freed.
+TWB_API int twb_trace_reduce_add_rms_norm(const void* const* partials, int num_partials, void* y, void* residual,
                                          const void* weight, int64_t num_tokens, int64_t hidden_size,
                                          int max_ctas, float epsilon, void* trace, void* stream) {
   if (!trace) return tw::set_error(TW_ERR_INVALID_ARGUMENT, "trace: null trace buffer");
   unsigned long long* buf = static_cast<unsigned long long*>(trace);
-  static unsigned long long* current = nullptr;  // bench.py calls from one thread, on one device
-  if (buf != current) {
+  if (buf != twb::g_trace_current) {  // bench.py calls from one thread, on one device
     if (hipMemcpyToSymbol(HIP_SYMBOL(tw::g_trace), &buf, sizeof(buf)) != hipSuccess)
       return tw::set_error(TW_ERR_LAUNCH, "trace: could not set the trace pointer");
-    current = buf;
+    twb::g_trace_current = buf;
   }
   return tw::run_row_norm("trace_reduce_add_rms_norm", partials, num_partials, y, residual, nullptr, weight,
                           nullptr, num_tokens, hidden_size, epsilon, TW_DTYPE_BF16, max_ctas, true, stream);
 }
 
+
+// Ends a traced burst: kernels launched after this write no stamps (the trace buffer may
+// be freed).  Synchronous.
+TWB_API int twb_trace_end(void) {
+  unsigned long long* none = nullptr;
+  if (hipMemcpyToSymbol(HIP_SYMBOL(tw::g_trace), &none, sizeof(none)) != hipSuccess)
+    return tw::set_error(TW_ERR_LAUNCH, "trace: could not clear the trace pointer");
+  twb::g_trace_current = nullptr;
+  return TW_OK;
+}
+
+TWB_API const char* twb_last_error(void) { return tw_last_error(); }
+
+// tw_reduce_add_rms_norm_ws through the split-row kernel with `segs_nwaves` waves per
+// segment (4 or 8), the segments of a row placed on CONSECUTIVE workgroups — hence on
+// different XCDs — instead of on one XCD: the form the product does not launch.  Requires
+// what the split-row kernel requires (bf16, 16-byte alignment, hidden_size % 8 == 0,
+// 1 <= num_tokens <= TW_SPLIT_MAX_TOKENS, a zeroed 256-byte aligned workspace of
+// TW_SPLIT_WORKSPACE_BYTES) and at least two segments per row.
+TWB_API int twb_reduce_add_rms_norm_split_spread(const void* const* partials, int num_partials, void* y,
+                                                 void* residual, const void* weight, int64_t num_tokens,
+                                                 int64_t hidden_size, float epsilon, int seg_waves,
+                                                 void* workspace, void* stream) {
+  const char* what = "reduce_add_rms_norm_split_spread";
+  if (!partials || !y || !residual || !weight || !workspace || num_partials < 1 || num_partials > TW_MAX_PARTIALS ||
+      num_tokens < 1 || num_tokens > TW_SPLIT_MAX_TOKENS || hidden_size < 8 || hidden_size % 8 != 0 ||
+      (seg_waves != 4 && seg_waves != 8))
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "%s: bad argument", what);
+  const int V = (int)(hidden_size / 8);
+  const int nchunks = (V + 63) / 64;
+  const int segs = (nchunks + seg_waves - 1) / seg_waves;
+  if (nchunks > tw::kMaxChunks || segs < 2)
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "%s: the row has %d chunks, need 2 .. %d segments' worth", what,
+                         nchunks, tw::kMaxChunks);
+  auto misaligned = [](const void* p, unsigned n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) != 0; };
+  tw::PartialPtrs parts = {};
+  bool bad = misaligned(y, 16) || misaligned(residual, 16) || misaligned(weight, 16) || misaligned(workspace, 256);
+  for (int p = 0; p < num_partials; ++p) {
+    if (!partials[p]) return tw::set_error(TW_ERR_INVALID_ARGUMENT, "%s: partial %d is null", what, p);
+    bad = bad || misaligned(partials[p], 16);
+    parts.p[p] = partials[p];
+  }
+  if (bad) return tw::set_error(TW_ERR_ALIGNMENT, "%s: misaligned pointer", what);
+  const dim3 g((unsigned)(num_tokens * segs)), b((unsigned)(seg_waves * 64));
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  tw::SplitRow* ws = static_cast<tw::SplitRow*>(workspace);
+#define TWB_SPREAD(NP)                                                                                          \
+  tw::launch_kernel(tw::row_norm_split_kernel<NP, false>, g, b, 0, hs, parts, num_partials, y, residual, weight, \
+                    ws, epsilon, (int)num_tokens, V, (float)hidden_size, segs, seg_waves * 64)
+  switch (num_partials) {
+    case 1: TWB_SPREAD(1); break;
+    case 2: TWB_SPREAD(2); break;
+    case 4: TWB_SPREAD(4); break;
+    case 8: TWB_SPREAD(8); break;
+    default: TWB_SPREAD(0); break;
+  }
+#undef TWB_SPREAD
+  return tw::finish_launch(what);
+}
 
 static int bench_lds_limit(const void* fn, int bytes) {
   return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess ? TW_OK
@@ -386,7 +480,7 @@ static int bench_lds_limit(const void* fn, int bytes) {
 
 // The GEMM's k loop from its parts (see gemm_loop_kernel).  src: 8 * window bytes of device
 // memory, window a power of two >= 128 KiB; out: 2 * grid int64; sink: 512 floats.
-TW_API int twb_gemm_loop(int slabs, int parts, int64_t window, const void* src, void* out, void* sink, int grid,
+TWB_API int twb_gemm_loop(int slabs, int parts, int64_t window, const void* src, void* out, void* sink, int grid,
                          void* stream) {
   if (slabs < 1 || grid < 1 || !src || !out || !sink || window < (128 << 10) || window > (1ll << 30) ||
       (window & (window - 1)))
@@ -399,7 +493,7 @@ TW_API int twb_gemm_loop(int slabs, int parts, int64_t window, const void* src, 
 }
 
 // src: 1 MiB of device memory; out: grid int64; sink: 1024 uint32.
-TW_API int twb_lds_read_rate(int iters, int waves, int dma, const void* src, void* out, void* sink, int grid,
+TWB_API int twb_lds_read_rate(int iters, int waves, int dma, const void* src, void* out, void* sink, int grid,
                              void* stream) {
   if (iters < 1 || waves < 1 || waves > 16 || grid < 1 || !src || !out || !sink)
     return tw::set_error(TW_ERR_INVALID_ARGUMENT, "lds_read_rate: bad argument");

@@ -30,7 +30,11 @@
 extern "C" {
 #endif
 
+/* Exported from the shared library.  (A build that compiles the sources into another
+ * library may define TW_API beforehand to keep these names out of its own exports.) */
+#ifndef TW_API
 #define TW_API __attribute__((visibility("default")))
+#endif
 
 #define TW_OK 0
 #define TW_ERR_INVALID_ARGUMENT (-1) /* null pointer, negative size, bad P / rank */
@@ -205,6 +209,17 @@ TW_API int tw_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M,
                     int64_t N, int64_t K, int64_t ldc, int max_cus,
                     void* stream);
 
+/* tw_gemm_bf16_nt with the linear layer's optional bias: bias is [N] bf16 in device
+ * memory (8-byte aligned) or NULL.  It is added as the reference adds it — to the
+ * product already rounded to bf16, in fp32, rounded again:
+ *   out = bf16_rne( f32(bf16_rne(a * b^T)) + f32(bias) )
+ * (torch.matmul(x, W.t(), out=output); output += bias,
+ * vllm/model_executor/layers/linear.py:224-228).  In a tensor-parallel layer only
+ * rank 0 passes its bias (linear.py:1306-1308), so the P-way sum holds it once. */
+TW_API int tw_gemm_bf16_nt_bias(void* out, const void* a, const void* b, const void* bias,
+                         int64_t M, int64_t N, int64_t K, int64_t ldc, int max_cus,
+                         void* stream);
+
 /* The producer of the fused op's input: the P row-parallel partial sums of one
  * token split in ONE launch, outs[p][M, N] = as[p][M, K] * bs[p][N, K]^T for
  * p < num_partials, each written straight into its rank's staging rows (outs[p] =
@@ -282,6 +297,15 @@ TW_API int tw_reduce_add_rms_norm_dynamic_per_token_quant(
     const void* const* partials, int num_partials, void* out, float* scales, void* residual,
     const void* weight, const float* scale_ub, int64_t num_tokens, int64_t hidden_size,
     int max_ctas, float epsilon, int out_kind, void* stream);
+
+/* tw_gemm_bf16_nt_partials with a bias per product: biases is NULL or a HOST array of
+ * num_partials device pointers, each [N] bf16 or NULL (one GPU standing in for the ranks
+ * passes rank 0's bias in biases[0] and NULL elsewhere, linear.py:1306-1308).  Same
+ * arithmetic as tw_gemm_bf16_nt_bias; bit-identical to num_partials calls of it. */
+TW_API int tw_gemm_bf16_nt_partials_bias(void* const* outs, const void* const* as,
+                                  const void* const* bs, const void* const* biases,
+                                  int num_partials, int64_t M, int64_t N, int64_t K,
+                                  int64_t ldc, int max_cus, void* stream);
 
 #ifdef __cplusplus
 }

@@ -49,3 +49,20 @@ def assert_parity(y_got, r_got, y_want, r_want, what: str, max_y_ulp=1, max_y_mi
     assert d.max() <= max_y_ulp, f"{what}: y off by {d.max()} ulp"
     frac = float((d != 0).mean())
     assert frac <= max_y_mismatch, f"{what}: {frac:.2%} of y elements differ by an ulp"
+
+
+def bench_lib():
+    """benchlib/libtw_bench.so (measurement and test-only kernels), or a skip when it has
+    not been built.  Its error text comes from twb_last_error()."""
+    import ctypes
+    import os
+
+    import pytest
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "benchlib", "libtw_bench.so")
+    if not os.path.exists(path):
+        pytest.skip(f"{path} has not been built (make -C benchlib)")
+    L = ctypes.CDLL(path)
+    vp, i64, ci, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+    L.twb_last_error.restype = ctypes.c_char_p
+    L.twb_reduce_add_rms_norm_split_spread.argtypes = [ctypes.POINTER(vp), ci, vp, vp, vp, i64, i64, f32, ci, vp, vp]
+    return L

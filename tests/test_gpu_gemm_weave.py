@@ -243,3 +243,162 @@ def test_weave_step_equals_serial_execution():
         torch.cuda.synchronize()
         assert torch.equal(buf1.storage, buf2.storage) and torch.equal(res1, res2)
     check(buf2.local[:Ta], g.a, g.b, "weave gemm split")
+
+
+# ---------------------------------------------------------------------------
+# bias of the in-place linear (vllm/model_executor/layers/linear.py:224-228) and the
+# RowParallelLinear call surface (linear.py:1290-1334)
+# ---------------------------------------------------------------------------
+def reference_linear_inplace(a, b, bias):
+    """The reference's two steps on the CPU: the product rounded to bf16
+    (torch.matmul(..., out=bf16)), then `output += bias` in bf16 arithmetic (fp32 add, one
+    more rounding).  The product is taken from `a @ b.T` in fp32."""
+    prod = (a.float().cpu() @ b.float().cpu().t()).to(torch.bfloat16)
+    return prod if bias is None else (prod.float() + bias.float().cpu()).to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("M,N,K,ldc,shift", [
+    (100, 128, 64, 128, 0),          # fallback kernel
+    (129, 256, 72, 256, 0),          # fallback kernel, K % 64 != 0
+    (300, 384, 128, 384, 0),         # big kernel, 16-byte stores
+    (300, 388, 128, 388, 0),         # big kernel, 8-byte stores (N % 8 != 0)
+    (300, 384, 128, 384, 4),         # big kernel, out not 16-byte aligned
+    (2458, 8192, 1024, 8192, 0),     # config 5's shape
+    (2048, 10240, 128, 10240, 0),    # 256 x 384 tiles
+])
+def test_gemm_bias_matches_the_reference_two_step_arithmetic(M, N, K, ldc, shift):
+    """out = bf16(bf16(a b^T) + bias): against fp32 CPU arithmetic within the path's
+    tolerance, and BIT-identical to adding the bias in bf16 to the library's own
+    bias-free product — the reference's `output += bias` on top of its matmul."""
+    print(f"[case] gemm bias M={M} N={N} K={K} ldc={ldc} shift={shift}", flush=True)
+    g = wl.make_gemm_inputs(M, N, K, DEV, seed=M + N + K + shift)
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(M * 31 + N)
+    bias = torch.randn(N, generator=gen, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    flat = torch.zeros(M * ldc + 16, dtype=torch.bfloat16, device=DEV)
+    out = flat[shift:shift + M * ldc].view(M, ldc)[:, :N]
+    plain = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16_nt(out, g.a, g.b, bias=bias)
+    ops.gemm_bf16_nt(plain, g.a, g.b)
+    torch.cuda.synchronize()
+    assert torch.equal(out, plain + bias), "fused bias differs from `output += bias` on the bias-free product"
+    want = reference_linear_inplace(g.a, g.b, bias)
+    torch.testing.assert_close(out.float().cpu(), want.float(), rtol=RTOL, atol=ATOL)
+    assert not flat[:shift].any() and not flat[shift + M * ldc:].any()
+
+
+def test_gemm_bias_argument_checks():
+    g = wl.make_gemm_inputs(64, 128, 64, DEV, seed=3)
+    out = torch.empty((64, 128), dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="bias has shape"):
+        ops.gemm_bf16_nt(out, g.a, g.b, bias=torch.zeros(64, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(RuntimeError, match="dtype"):
+        ops.gemm_bf16_nt(out, g.a, g.b, bias=torch.zeros(128, dtype=torch.float32, device=DEV))
+    odd = torch.zeros(130, dtype=torch.bfloat16, device=DEV)[1:129]   # 2-byte aligned only
+    with pytest.raises(RuntimeError, match="aligned"):
+        ops.gemm_bf16_nt(out, g.a, g.b, bias=odd)
+
+
+def test_partials_producer_adds_only_rank_zero_bias():
+    """One GPU standing in for the ranks: biases = [b, None, ...] puts the bias into slot 0
+    only, bit-identical to per-rank calls, so the P-way sum holds it once."""
+    P, M, N, K = 4, 333, 512, 128
+    gs = wl.make_partials_gemm_inputs(P, M, N, K, DEV, seed=77)
+    bias = torch.linspace(-2, 2, N, device=DEV).to(torch.bfloat16)
+    buf = tw.PartialsBuffer(P, M, N, rank=0, device=DEV)
+    ops.gemm_bf16_nt_partials([buf.slot(p)[:M] for p in range(P)], [g.a for g in gs], [g.b for g in gs],
+                              biases=[bias] + [None] * (P - 1))
+    torch.cuda.synchronize()
+    for p in range(P):
+        one = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+        ops.gemm_bf16_nt(one, gs[p].a, gs[p].b, bias=bias if p == 0 else None)
+        torch.cuda.synchronize()
+        assert torch.equal(buf.slot(p)[:M], one), f"slot {p}"
+
+
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_row_parallel_linear_tokenweave_call_site(oracle, with_bias):
+    """llama.py:248-249 on one GPU: every rank's o_proj writes its partial sum in place into
+    its staging rows (`forward(x_p, output_=rows, is_tokenweave=True)`), the fused norm
+    reduces them.  Against fp32 `x @ W.T + b` per rank, and against the CPU checker fed
+    with the staged partials."""
+    ws, T, H, Kfull = 4, 200, 1024, 1024
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(91 + with_bias)
+    W = (torch.randn(H, Kfull, generator=gen, device=DEV) * 0.03).to(torch.bfloat16)
+    b = torch.randn(H, generator=gen, device=DEV).to(torch.bfloat16)
+    x = torch.randn(T, Kfull, generator=gen, device=DEV).to(torch.bfloat16)
+    buf = tw.PartialsBuffer(ws, T, H, rank=0, device=DEV)
+    layers = []
+    for p in range(ws):
+        lin = tw.RowParallelLinear(Kfull, H, bias=with_bias, tp_rank=p, tp_size=ws).to(DEV)
+        lin.weight_loader(lin.weight, W)
+        if with_bias:
+            lin.weight_loader(lin.bias, b)
+        layers.append(lin)
+        shard = Kfull // ws
+        xp = x[:, p * shard:(p + 1) * shard].contiguous()
+        out, out_bias = lin(xp, buf.slot(p)[:T], is_tokenweave=True)
+        assert out.data_ptr() == buf.slot(p).data_ptr() and out_bias is None
+        torch.cuda.synchronize()
+        want = xp.float().cpu() @ lin.weight.data.float().cpu().t()
+        if with_bias and p == 0:
+            want = want + b.float().cpu()
+        torch.testing.assert_close(out.float().cpu(), want, rtol=RTOL, atol=ATOL)
+    # input_is_parallel=False slices the full activation itself
+    lin = tw.RowParallelLinear(Kfull, H, bias=False, input_is_parallel=False, tp_rank=2, tp_size=ws).to(DEV)
+    lin.weight_loader(lin.weight, W)
+    out2 = torch.empty((T, H), dtype=torch.bfloat16, device=DEV)
+    lin(x, out2, is_tokenweave=True)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, buf.slot(2)[:T])
+    # the fused op on the staged partials
+    parts = [to_bits(buf.slot(p)[:T]) for p in range(ws)]
+    res = torch.randn(T, H, generator=gen, device=DEV).to(torch.bfloat16)
+    res_bits = to_bits(res)
+    norm = tw.RMSNorm(H, eps=1e-5, dtype=torch.bfloat16).to(DEV)
+    tw.fused_allreduce_layernorm(norm, buf.hidden_states(T), res, buf, T // ws, 0, ws, 0, row_range=(0, T))
+    torch.cuda.synchronize()
+    y_w, r_w = oracle.reduce_add_rms_norm(parts, res_bits, to_bits(norm.weight.data), 1e-5)
+    assert np.array_equal(to_bits(res), r_w)
+    f = lambda u: (u.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    assert np.all(np.abs(f(to_bits(buf.hidden_states(T))) - f(y_w)) <= ATOL + RTOL * np.abs(f(y_w)))
+
+
+def test_row_parallel_linear_default_mode_and_skip_bias_add():
+    T, H, K = 64, 256, 128
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(17)
+    x = torch.randn(T, K, generator=gen, device=DEV).to(torch.bfloat16)
+    lin = tw.RowParallelLinear(K, H, bias=True, skip_bias_add=True).to(DEV)
+    lin.weight.data.copy_((torch.randn(H, K, generator=gen, device=DEV) * 0.05).to(torch.bfloat16))
+    lin.bias.data.copy_(torch.randn(H, generator=gen, device=DEV).to(torch.bfloat16))
+    out, out_bias = lin(x)                      # default mode, tp_size 1: a fresh output, bias handed back
+    torch.cuda.synchronize()
+    assert out_bias is lin.bias
+    torch.testing.assert_close(out.float().cpu(), x.float().cpu() @ lin.weight.data.float().cpu().t(),
+                               rtol=RTOL, atol=ATOL)
+    with pytest.raises(AssertionError, match="preallocated"):
+        lin(x, None, is_tokenweave=True)
+    multi = tw.RowParallelLinear(K * 2, H, bias=False, tp_rank=1, tp_size=2).to(DEV)
+    with pytest.raises(RuntimeError, match="no collectives"):
+        multi(x)
+
+
+def test_tuner_returns_a_well_formed_table():
+    """tune() on one small token count, two offsets, few rounds: the table has the layout
+    load_config / weave_plan read, and the budgets come from the measured grid."""
+    from tokenweave_amd import tune_weave
+    lines = []
+    table = tune_weave.tune(2048, 256, 4, [1024], offsets=(0, 128), device=DEV, log=lines.append, k_mlp=512,
+                            regions=2, stage_budget_us=300.0)
+    assert set(table) == {"1024"}
+    e = table["1024"]
+    assert set(e) == {"attention_ctas", "mlp_ctas", "split_offset", "gemm_cus", "mlp_gemm_cus", "overlap"}
+    cus = ops.num_compute_units(DEV)
+    assert e["split_offset"] in (0, 128) and e["overlap"] in (0, 1)
+    assert e["attention_ctas"] in (0, cus // 2) and e["mlp_ctas"] in (0, cus // 2)
+    assert 0 <= e["gemm_cus"] <= cus and 0 <= e["mlp_gemm_cus"] <= cus
+    assert any("split_offset=" in ln for ln in lines)
+    plan = tw.weave_plan(1024, {1024: e})
+    assert plan is None or plan["split_size"] == tw.tokenweave_split_size(1024, e["split_offset"])

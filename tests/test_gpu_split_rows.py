@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import tokenweave_amd as tw
-from helpers import assert_parity, to_bits
+from helpers import assert_parity, bench_lib, to_bits
 from tokenweave_amd import _custom_ops as ops
 from tokenweave_amd import _lib
 from tokenweave_amd import workloads as wl
@@ -132,6 +132,99 @@ def test_graph_capture_and_replay_of_the_split_kernel():
         g.replay()
         torch.cuda.synchronize()
         assert np.array_equal(to_bits(out), want[0]) and np.array_equal(to_bits(res), want[1])
+
+
+def run_spread(L, inp, seg_waves, ws, alias=0):
+    """The split-row kernel with the segments of a row on consecutive workgroups, i.e. on
+    different XCDs (the measurement library's form; the product keeps a row on one XCD)."""
+    cfg = inp.cfg
+    parts = [p.clone() for p in inp.partials]
+    res = inp.residual.clone()
+    out = parts[alias] if alias is not None else torch.empty_like(res)
+    ptrs = (ctypes.c_void_p * cfg.P)(*[p.data_ptr() for p in parts])
+    rc = L.twb_reduce_add_rms_norm_split_spread(ptrs, cfg.P, out.data_ptr(), res.data_ptr(), inp.weight.data_ptr(),
+                                                cfg.T, cfg.H, cfg.eps, seg_waves, ws.data_ptr(),
+                                                torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, L.twb_last_error().decode()
+    torch.cuda.synchronize()
+    return to_bits(out), to_bits(res)
+
+
+@pytest.mark.parametrize("seg_waves", [4, 8])
+@pytest.mark.parametrize("T,P,H", [(1, 8, 8192), (8, 8, 8192), (32, 8, 8192), (32, 1, 8192), (48, 8, 8192),
+                                   (3, 3, 8200), (7, 5, 12288), (9, 16, 8192), (40, 4, 16384), (5, 7, 32768),
+                                   (47, 2, 16392), (256, 8, 8192), (2, 2, 1024)])
+def test_segments_spread_over_xcds_bit_identical(T, P, H, seg_waves):
+    """The hand-over between the segment workgroups of a row does not depend on their
+    sharing an XCD: with the segments of every row spread over the XCDs the results are the
+    one-workgroup kernel's, bit for bit, five launches in a row on one workspace."""
+    L = bench_lib()
+    if (H // 8 + 63) // 64 <= seg_waves:
+        pytest.skip("the row is a single segment of this size")
+    print(f"[case] spread split T={T} P={P} H={H} waves per segment={seg_waves}", flush=True)
+    cfg, inp = make(P, T, H, seed=71)
+    want = run(inp, False, alias=P - 1)
+    ws = torch.zeros(_lib.TW_SPLIT_WORKSPACE_BYTES, dtype=torch.uint8, device=DEV)
+    for i in range(5):
+        got = run_spread(L, inp, seg_waves, ws, alias=P - 1)
+        assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]), f"launch {i}"
+    assert int(ws.view(torch.int32).view(-1, 96)[:, 64].abs().max()) == 0, "an arrival counter was left non-zero"
+
+
+@pytest.mark.parametrize("form,launches", [("product", 3072), ("spread", 1536)])
+def test_soak_alternating_decode_shapes_on_one_workspace(form, launches):
+    """A few thousand back-to-back launches of the split-row kernel on ONE workspace,
+    alternating between the decode shapes (1 .. 48 rows, hidden size 8192 / 16384, one and
+    eight partials), every result compared with the one-workgroup kernel's bits on the GPU.
+    The launches of a block of 128 are not separated by host synchronisation (the next
+    launch follows as closely as the queue allows, which is when a stale value left by the
+    previous one would be seen); the run stops at the first block that holds a mismatch and
+    names its first launch."""
+    L = bench_lib() if form == "spread" else None
+    shapes = [(T, P, H) for H in (8192, 16384) for P in (1, 8) for T in (1, 8, 32, 48)]
+    ws = torch.zeros(_lib.TW_SPLIT_WORKSPACE_BYTES, dtype=torch.uint8, device=DEV)
+    cases = []
+    for i, (T, P, H) in enumerate(shapes):
+        assert ops.split_segments(T, H) > 1
+        cfg, inp = make(P, T, H, seed=300 + i)
+        y_w, r_w = run(inp, False, alias=None)
+        res = inp.residual.clone()
+        out = torch.empty_like(res)
+        ptrs = (ctypes.c_void_p * P)(*[p.data_ptr() for p in inp.partials])
+        cases.append(dict(cfg=cfg, inp=inp, res=res, out=out, ptrs=ptrs,
+                          y_want=torch.from_numpy(y_w.view(np.int16)).to(DEV),
+                          r_want=torch.from_numpy(r_w.view(np.int16)).to(DEV)))
+    lib = _lib.lib()
+    sp = torch.cuda.current_stream().cuda_stream
+    block = 128
+    flags = torch.zeros(block, dtype=torch.int32, device=DEV)
+    rng = np.random.default_rng(5)
+    order = rng.integers(0, len(cases), size=launches)
+    for b0 in range(0, launches, block):
+        flags.zero_()
+        for j, ci in enumerate(order[b0:b0 + block]):
+            c = cases[ci]
+            cfg = c["cfg"]
+            c["res"].copy_(c["inp"].residual)
+            if form == "spread":
+                rc = L.twb_reduce_add_rms_norm_split_spread(c["ptrs"], cfg.P, c["out"].data_ptr(),
+                                                            c["res"].data_ptr(), c["inp"].weight.data_ptr(), cfg.T,
+                                                            cfg.H, cfg.eps, 4 if ci % 2 else 8, ws.data_ptr(), sp)
+                assert rc == 0, L.twb_last_error().decode()
+            else:
+                rc = lib.tw_reduce_add_rms_norm_ws(c["ptrs"], cfg.P, c["out"].data_ptr(), c["res"].data_ptr(),
+                                                   c["inp"].weight.data_ptr(), cfg.T, cfg.H, 0, cfg.eps,
+                                                   ws.data_ptr(), ws.numel(), sp)
+                assert rc == 0, _lib.last_error()
+            bad = (c["out"].view(torch.int16) != c["y_want"]).any() | (c["res"].view(torch.int16) != c["r_want"]).any()
+            flags[j] = bad.to(torch.int32)
+        f = flags.cpu().numpy()
+        if f.any():
+            j = int(np.flatnonzero(f)[0])
+            T, P, H = shapes[order[b0 + j]]
+            pytest.fail(f"{form}: launch {b0 + j} (T={T} P={P} H={H}) differs from the one-workgroup kernel; "
+                        f"{int(f.sum())} of the block's {len(f)} launches differ")
+    assert int(ws.view(torch.int32).view(-1, 96)[:, 64].abs().max()) == 0, "an arrival counter was left non-zero"
 
 
 def test_workspace_argument_checks():

@@ -265,3 +265,24 @@ def test_weave_plan_honours_measured_no_overlap_entries():
     shipped = tw.load_config()
     assert all("overlap" in e for e in shipped.values())
     assert tw.weave_plan(16384, shipped) is not None
+
+
+def test_row_parallel_linear_constructor_contract():
+    """Constructor checks of RowParallelLinear (vllm/model_executor/layers/linear.py:1185-1240):
+    shapes per rank, the reduce_results / bias guard, rank bounds."""
+    import tokenweave_amd as tw
+    lin = tw.RowParallelLinear(8192, 8192, bias=True, tp_rank=3, tp_size=8)
+    assert tuple(lin.weight.shape) == (8192, 1024) and tuple(lin.bias.shape) == (8192,)
+    assert lin.weight.dtype == torch.bfloat16 and lin.input_size_per_partition == 1024
+    assert "tp_size=8" in lin.extra_repr() and "input_features=1024" in lin.extra_repr()
+    assert tw.RowParallelLinear(64, 64, bias=False).bias is None
+    with pytest.raises(ValueError, match="When not reduce the results"):
+        tw.RowParallelLinear(64, 64, bias=True, reduce_results=False)
+    with pytest.raises(ValueError, match="Invalid rank"):
+        tw.RowParallelLinear(64, 64, tp_rank=2, tp_size=2)
+    with pytest.raises(ValueError, match="not divisible"):
+        tw.RowParallelLinear(100, 64, tp_size=8)
+    full = torch.arange(64 * 64, dtype=torch.float32).view(64, 64).to(torch.bfloat16)
+    lin = tw.RowParallelLinear(64, 64, bias=False, tp_rank=1, tp_size=4)
+    lin.weight_loader(lin.weight, full)
+    assert torch.equal(lin.weight.data, full[:, 16:32])

@@ -7,11 +7,12 @@ reference's op shims (``vllm/_custom_ops.py:176-221``), its ``RMSNorm`` layer
 """
 from . import _custom_ops as ops  # noqa: F401
 from .layernorm import RMSNorm  # noqa: F401
+from .linear import RowParallelLinear, UnquantizedLinearMethod  # noqa: F401
 from .tokenweave_utils import (PartialsBuffer, fused_allreduce_layernorm,  # noqa: F401
                                load_config, select_config, shard_bounds, tokenweave_split_size,
                                tokenweave_overlap, tokenweave_with_fuse_only,
                                weave_norm_gemm, weave_plan)
 
-__all__ = ["ops", "RMSNorm", "PartialsBuffer", "fused_allreduce_layernorm", "shard_bounds",
+__all__ = ["ops", "RMSNorm", "RowParallelLinear", "UnquantizedLinearMethod", "PartialsBuffer", "fused_allreduce_layernorm", "shard_bounds",
            "tokenweave_split_size", "tokenweave_with_fuse_only", "tokenweave_overlap", "weave_norm_gemm", "load_config", "select_config", "weave_plan"]
 __version__ = "0.1.0"

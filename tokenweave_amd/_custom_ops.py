@@ -19,6 +19,7 @@ import itertools
 import os
 import types
 import threading
+import warnings
 import weakref
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -38,8 +39,12 @@ _DTYPE_CODE = {torch.bfloat16: _lib.TW_DTYPE_BF16, torch.float16: _lib.TW_DTYPE_
 BINDING_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtokenweave_amd_torch.so")
 COMPILED_BINDING = False
 if os.path.exists(BINDING_PATH) and os.environ.get("TOKENWEAVE_AMD_NO_COMPILED_BINDING") != "1":
-    torch.ops.load_library(BINDING_PATH)
-    COMPILED_BINDING = True
+    try:
+        torch.ops.load_library(BINDING_PATH)
+        COMPILED_BINDING = True
+    except OSError as e:   # e.g. built against another torch: the ctypes route serves every op
+        warnings.warn(f"{BINDING_PATH} could not be loaded ({e}); tokenweave_amd registers its ops "
+                      "from Python and calls the HIP library through ctypes instead", RuntimeWarning)
 _T = torch.ops.tokenweave_amd
 
 # Message of the reference's launchers (csrc/tokenweave_fused_kernels.cu:259).
@@ -290,18 +295,44 @@ def _peer_stride(mcptr: int, world_size: int, nbytes: int) -> int:
 # --- workspace of the split-row kernel (decode-size batches) -------------------
 # One zeroed TW_SPLIT_WORKSPACE_BYTES buffer per (device, stream): calls on one stream
 # are ordered, which is what sharing a workspace requires.  Allocated on the first
-# small-batch call on that stream and kept for the life of the process.
+# small-batch call on that stream — never while the stream is being captured into a
+# graph — and kept for the life of the process.
 _SPLIT_WS: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
-def split_workspace(device_index: int, stream_ptr: int) -> torch.Tensor:
+def split_workspace(device_index: int, stream_ptr: int) -> Optional[torch.Tensor]:
+    """The workspace of (device, stream), made on first use.  While the stream is being
+    captured nothing is allocated (the buffer would come out of the graph's private pool
+    and its fill kernel would be recorded): without a workspace made beforehand
+    (`prepare_split_workspace`, or any eager decode-size call on that stream) the caller
+    gets None and runs the one-workgroup-per-row kernel, whose results are the same bits."""
     ws = _SPLIT_WS.get((device_index, stream_ptr))
     if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None
         ws = torch.zeros(_lib.TW_SPLIT_WORKSPACE_BYTES, dtype=torch.uint8,
                          device=torch.device("cuda", device_index))
         assert ws.data_ptr() % 256 == 0
         _SPLIT_WS[(device_index, stream_ptr)] = ws
     return ws
+
+
+def prepare_split_workspace(device=None, stream: Optional[torch.cuda.Stream] = None) -> None:
+    """Create the split-row workspace of `stream` (default: the current stream of `device`)
+    now.  Call it before capturing decode-size calls of `fused_rs_ln_ag_cta` /
+    `fused_rs_ln_cta` / `reduce_add_rms_norm` on that stream into a HIP graph
+    (`torch.cuda.graph(g, stream=stream)`): a capture never allocates, and without the
+    workspace those calls record the one-workgroup-per-row kernel (same results, up to
+    0.8 us slower per call).  A graph's split-row nodes use the capture stream's workspace:
+    graphs captured on one stream must not be replayed concurrently on different streams."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    if COMPILED_BINDING:
+        with torch.cuda.device(idx), torch.cuda.stream(stream or torch.cuda.current_stream(idx)):
+            _T.prepare_split_workspace(idx)
+    sp = (stream or torch.cuda.current_stream(idx)).cuda_stream
+    with torch.cuda.device(idx):
+        split_workspace(idx, sp)
 
 
 def _wants_split(T: int, cap: int) -> bool:
@@ -323,9 +354,11 @@ def _fused_rs_ln(entry: str, kname: str, input, residual, weight, mcptr, signal_
     cap = _cap(MAX_CTAS)
     with _on_device(input):
         sp = _stream_ptr(input)
+        ws = None
         if _wants_split(T, cap):
             idx = input.device.index
             ws = split_workspace(torch.cuda.current_device() if idx is None else idx, sp)
+        if ws is not None:
             _lib.check(_lib.lib().tw_fused_rs_ln_ag_cta_ws(
                 input.data_ptr(), residual.data_ptr(), weight.data_ptr(), int(mcptr), stride,
                 int(rank), int(world_size), cap, epsilon, T, H, ws.data_ptr(), ws.numel(), sp))
@@ -415,8 +448,10 @@ def reduce_add_rms_norm(partials: Sequence[torch.Tensor], out: torch.Tensor,
     L = _lib.lib()
     with _on_device(out):
         sp = _stream_ptr(out)
+        ws = None
         if _wants_split(T, cap) if split is None else split:
             ws = split_workspace(dev.index if dev.index is not None else torch.cuda.current_device(), sp)
+        if ws is not None:
             rc = L.tw_reduce_add_rms_norm_ws(ptrs, P, out.data_ptr(), residual.data_ptr(), weight.data_ptr(), T, H,
                                              cap, epsilon, ws.data_ptr(), ws.numel(), sp)
         else:
@@ -620,7 +655,14 @@ def reduce_add_rms_norm_dynamic_per_token_quant(partials: Sequence[torch.Tensor]
             _stream_ptr(first)))
 
 
-def _prepare_gemm_bf16_nt(out, a, b, max_cus):
+def _check_bias(bias, N, dev):
+    if bias is None:
+        return
+    _check_tensor("bias", bias, torch.bfloat16, dev)
+    _require(bias.dim() == 1 and bias.numel() == N, f"bias has shape {tuple(bias.shape)}, expected {(N,)}")
+
+
+def _prepare_gemm_bf16_nt(out, a, b, max_cus, bias=None):
     _require_bf16("gemm_bf16_nt_kernel", a)
     dev = a.device
     _check_tensor("a", a, torch.bfloat16, dev)
@@ -633,58 +675,73 @@ def _prepare_gemm_bf16_nt(out, a, b, max_cus):
     _require(K == K2, f"inner dimensions differ: a is {tuple(a.shape)}, b is {tuple(b.shape)}")
     _require(tuple(out.shape) == (M, N), f"out has shape {tuple(out.shape)}, expected {(M, N)}")
     _require(out.stride(1) == 1 and (M <= 1 or out.stride(0) >= N), "out rows must be contiguous")
+    _check_bias(bias, N, dev)
     ldc = out.stride(0) if M > 1 else max(N, out.stride(0))
-    args = (out.data_ptr(), a.data_ptr(), b.data_ptr(), M, N, K, ldc, _cap(max_cus))
-    return _lib.lib().tw_gemm_bf16_nt, args, (out, a, b), dev
+    if bias is None:
+        args = (out.data_ptr(), a.data_ptr(), b.data_ptr(), M, N, K, ldc, _cap(max_cus))
+        return _lib.lib().tw_gemm_bf16_nt, args, (out, a, b), dev
+    args = (out.data_ptr(), a.data_ptr(), b.data_ptr(), bias.data_ptr(), M, N, K, ldc, _cap(max_cus))
+    return _lib.lib().tw_gemm_bf16_nt_bias, args, (out, a, b, bias), dev
 
 
 def gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
-                 max_cus: Optional[int] = None) -> None:
-    """out[M, N] <- a[M, K] @ b[N, K]^T (bf16, fp32 accumulate).  `out` may be a row
-    slice of a wider buffer (row stride >= N).  The in-place row-parallel linear of
+                 max_cus: Optional[int] = None, bias: Optional[torch.Tensor] = None) -> None:
+    """out[M, N] <- a[M, K] @ b[N, K]^T (bf16, fp32 accumulate), then `out += bias` as the
+    reference does it (on the rounded product, rounded again).  `out` may be a row slice of
+    a wider buffer (row stride >= N).  The in-place row-parallel linear of
     vllm/model_executor/layers/linear.py:203-228."""
-    BoundOp(*_prepare_gemm_bf16_nt(out, a, b, max_cus))()
+    BoundOp(*_prepare_gemm_bf16_nt(out, a, b, max_cus, bias))()
 
 
 def bind_gemm_bf16_nt(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor,
-                      max_cus: Optional[int] = None) -> BoundOp:
+                      max_cus: Optional[int] = None, bias: Optional[torch.Tensor] = None) -> BoundOp:
     """`gemm_bf16_nt` with the checks done now and the launch deferred."""
-    return BoundOp(*_prepare_gemm_bf16_nt(out, a, b, max_cus))
+    return BoundOp(*_prepare_gemm_bf16_nt(out, a, b, max_cus, bias))
 
 
-def _prepare_gemm_bf16_nt_partials(outs, a_list, b_list, max_cus):
+def _prepare_gemm_bf16_nt_partials(outs, a_list, b_list, max_cus, biases=None):
     P = len(outs)
     _require(1 <= P <= _lib.TW_MAX_PARTIALS, f"number of partials {P} not in [1, {_lib.TW_MAX_PARTIALS}]")
     _require(len(a_list) == P and len(b_list) == P, "outs, a and b must have one entry per partial")
+    _require(biases is None or len(biases) == P, "biases must have one entry (a tensor or None) per partial")
     shape = None
     for p in range(P):
         # the per-product checks of gemm_bf16_nt; all products must share one shape and row stride
-        _, args, _, dev = _prepare_gemm_bf16_nt(outs[p], a_list[p], b_list[p], max_cus)
+        _, args, _, dev = _prepare_gemm_bf16_nt(outs[p], a_list[p], b_list[p], max_cus,
+                                                None if biases is None else biases[p])
+        dims = args[-5:-1]
         if shape is None:
-            shape, dev0 = args[3:7], dev
-        _require(args[3:7] == shape and dev == dev0,
-                 f"partial {p} has (M, N, K, row stride) {args[3:7]}, partial 0 has {shape}")
+            shape, dev0 = dims, dev
+        _require(dims == shape and dev == dev0,
+                 f"partial {p} has (M, N, K, row stride) {dims}, partial 0 has {shape}")
     vp = ctypes.c_void_p
     o = (vp * P)(*[t.data_ptr() for t in outs])
     a = (vp * P)(*[t.data_ptr() for t in a_list])
     b = (vp * P)(*[t.data_ptr() for t in b_list])
-    args = (o, a, b, P, *shape, _cap(max_cus))
-    return _lib.lib().tw_gemm_bf16_nt_partials, args, (list(outs), list(a_list), list(b_list)), dev0
+    keep = (list(outs), list(a_list), list(b_list))
+    if biases is None or all(t is None for t in biases):
+        return _lib.lib().tw_gemm_bf16_nt_partials, (o, a, b, P, *shape, _cap(max_cus)), keep, dev0
+    bs = (vp * P)(*[None if t is None else t.data_ptr() for t in biases])
+    return (_lib.lib().tw_gemm_bf16_nt_partials_bias, (o, a, b, bs, P, *shape, _cap(max_cus)),
+            keep + (list(biases),), dev0)
 
 
 def gemm_bf16_nt_partials(outs: Sequence[torch.Tensor], a: Sequence[torch.Tensor], b: Sequence[torch.Tensor],
-                          max_cus: Optional[int] = None) -> None:
-    """outs[p][M, N] <- a[p][M, K] @ b[p][N, K]^T for every p in ONE launch: the P row-parallel
-    partial sums of a token split, each written straight into its rank's staging rows
-    (`outs[p]` = `PartialsBuffer.slot(p)[first_row:first_row + M]`).  The producer side of
-    the fused op: vllm/model_executor/layers/linear.py:203-228, 1310-1321."""
-    BoundOp(*_prepare_gemm_bf16_nt_partials(outs, a, b, max_cus))()
+                          max_cus: Optional[int] = None,
+                          biases: Optional[Sequence[Optional[torch.Tensor]]] = None) -> None:
+    """outs[p][M, N] <- a[p][M, K] @ b[p][N, K]^T (+ biases[p] where given) for every p in ONE
+    launch: the P row-parallel partial sums of a token split, each written straight into its
+    rank's staging rows (`outs[p]` = `PartialsBuffer.slot(p)[first_row:first_row + M]`).  The
+    producer side of the fused op: vllm/model_executor/layers/linear.py:203-228, 1310-1321
+    (only rank 0 adds its bias, :1306-1308: pass it as biases[0], None elsewhere)."""
+    BoundOp(*_prepare_gemm_bf16_nt_partials(outs, a, b, max_cus, biases))()
 
 
 def bind_gemm_bf16_nt_partials(outs: Sequence[torch.Tensor], a: Sequence[torch.Tensor],
-                               b: Sequence[torch.Tensor], max_cus: Optional[int] = None) -> BoundOp:
+                               b: Sequence[torch.Tensor], max_cus: Optional[int] = None,
+                               biases: Optional[Sequence[Optional[torch.Tensor]]] = None) -> BoundOp:
     """`gemm_bf16_nt_partials` with the checks done now and the launch deferred."""
-    return BoundOp(*_prepare_gemm_bf16_nt_partials(outs, a, b, max_cus))
+    return BoundOp(*_prepare_gemm_bf16_nt_partials(outs, a, b, max_cus, biases))
 
 
 def num_compute_units(device=None) -> int:

@@ -46,6 +46,7 @@ PROTOTYPES = {
     "tw_reduce_add_rms_norm_noalloc": [ctypes.POINTER(_vp), _ci, _vp, _vp, _vp, _i64, _i64, _ci, _f32, _vp],
     "tw_split_segments": [_i64, _i64, _ci],
     "tw_gemm_bf16_nt": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp],
+    "tw_gemm_bf16_nt_bias": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp],
     "tw_gemm_bf16_nt_partials": [ctypes.POINTER(_vp), ctypes.POINTER(_vp), ctypes.POINTER(_vp), _ci, _i64, _i64,
                                  _i64, _i64, _ci, _vp],
     "tw_rms_norm_static_fp8_quant": [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _ci, _vp],
@@ -55,6 +56,8 @@ PROTOTYPES = {
     "tw_rms_norm_dynamic_per_token_quant": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _ci, _ci, _vp],
     "tw_reduce_add_rms_norm_dynamic_per_token_quant": [ctypes.POINTER(_vp), _ci, _vp, _vp, _vp, _vp, _vp,
                                                        _i64, _i64, _ci, _f32, _ci, _vp],
+    "tw_gemm_bf16_nt_partials_bias": [ctypes.POINTER(_vp), ctypes.POINTER(_vp), ctypes.POINTER(_vp),
+                                      ctypes.POINTER(_vp), _ci, _i64, _i64, _i64, _i64, _ci, _vp],
 }
 
 _lib = None

@@ -263,13 +263,24 @@ int tw_reduce_add_rms_norm_dynamic_per_token_quant(const void* const* partials, 
 
 int tw_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t N, int64_t K,
                     int64_t ldc, int max_cus, void* stream) {
-  return tw::run_gemm_bf16_nt(out, a, b, M, N, K, ldc, max_cus, stream);
+  return tw::run_gemm_bf16_nt(out, a, b, nullptr, M, N, K, ldc, max_cus, stream);
+}
+
+int tw_gemm_bf16_nt_bias(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N,
+                         int64_t K, int64_t ldc, int max_cus, void* stream) {
+  return tw::run_gemm_bf16_nt(out, a, b, bias, M, N, K, ldc, max_cus, stream);
 }
 
 int tw_gemm_bf16_nt_partials(void* const* outs, const void* const* as, const void* const* bs,
                              int num_partials, int64_t M, int64_t N, int64_t K, int64_t ldc, int max_cus,
                              void* stream) {
-  return tw::run_gemm_bf16_nt_partials(outs, as, bs, num_partials, M, N, K, ldc, max_cus, stream);
+  return tw::run_gemm_bf16_nt_partials(outs, as, bs, nullptr, num_partials, M, N, K, ldc, max_cus, stream);
+}
+
+int tw_gemm_bf16_nt_partials_bias(void* const* outs, const void* const* as, const void* const* bs,
+                                  const void* const* biases, int num_partials, int64_t M, int64_t N,
+                                  int64_t K, int64_t ldc, int max_cus, void* stream) {
+  return tw::run_gemm_bf16_nt_partials(outs, as, bs, biases, num_partials, M, N, K, ldc, max_cus, stream);
 }
 
 }  // extern "C"

@@ -67,11 +67,14 @@ int run_row_norm_noalloc(const char* what, const void* const* partials, int np, 
 // (1 = the one-workgroup-per-row kernel runs instead).
 int split_segments(int64_t T, int64_t H, int max_ctas);
 
-int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t N,
+// bias: [N] bf16 added to every row of the product, or null.
+int run_gemm_bf16_nt(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N,
                      int64_t K, int64_t ldc, int max_cus, void* stream);
 
-int run_gemm_bf16_nt_partials(void* const* outs, const void* const* as, const void* const* bs, int count,
-                              int64_t M, int64_t N, int64_t K, int64_t ldc, int max_cus, void* stream);
+// biases: null, or `count` pointers each of which may be null.
+int run_gemm_bf16_nt_partials(void* const* outs, const void* const* as, const void* const* bs,
+                              const void* const* biases, int count, int64_t M, int64_t N, int64_t K,
+                              int64_t ldc, int max_cus, void* stream);
 
 }  // namespace tw
 

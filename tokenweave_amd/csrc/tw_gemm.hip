@@ -58,9 +58,19 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
+// The optional bias of the in-place linear is added the way the reference adds it
+// (vllm/model_executor/layers/linear.py:224-228: torch.matmul(..., out=output), then
+// output += bias): to the product already rounded to bf16, in fp32, rounded again.
+// `packed` and `bias2` hold two bf16 each, element 2i in the low half.
+__device__ __forceinline__ uint32_t add_bias2(uint32_t packed, uint32_t bias2) {
+  const float lo = __uint_as_float(packed << 16) + __uint_as_float(bias2 << 16);
+  const float hi = __uint_as_float(packed & 0xffff0000u) + __uint_as_float(bias2 & 0xffff0000u);
+  return pack2(lo, hi);
+}
+
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_nt_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
-    int M, int N, int K, int64_t ldc, int tiles_m, int tiles_n) {
+    const uint16_t* __restrict__ bias, int M, int N, int K, int64_t ldc, int tiles_m, int tiles_n) {
   __shared__ __attribute__((aligned(16))) uint16_t lds_a[2][BM * LDS_ROW];
   __shared__ __attribute__((aligned(16))) uint16_t lds_b[2][BN * LDS_ROW];
 
@@ -169,6 +179,11 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_nt_kernel(
             uint2 v;
             v.x = pack2(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1]);
             v.y = pack2(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+            if (bias) {  // N % 4 == 0: the four columns lie inside the row; bias is 8-byte aligned
+              const uint2 bv = *reinterpret_cast<const uint2*>(bias + n);
+              v.x = add_bias2(v.x, bv.x);
+              v.y = add_bias2(v.y, bv.y);
+            }
             *reinterpret_cast<uint2*>(out + (size_t)m * ldc + n) = v;
           }
         }
@@ -213,6 +228,7 @@ struct GemmBatch {
   uint16_t* out[TW_MAX_PARTIALS];
   const uint16_t* a[TW_MAX_PARTIALS];
   const uint16_t* b[TW_MAX_PARTIALS];
+  const uint16_t* bias[TW_MAX_PARTIALS];  // [N] bf16 or null: added to that product only
 };
 
 template <int TM, int TN>
@@ -256,6 +272,7 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
     const int product = pid / tiles_per_product;
     pid -= product * tiles_per_product;
     uint16_t* __restrict__ out = batch.out[product];
+    const uint16_t* __restrict__ bias = batch.bias[product];
     const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(batch.a[product]), 0, (uint32_t)((size_t)M * K * 2), 0x00020000);
     const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc(
@@ -411,6 +428,9 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
       const int rd_row = lane / CHUNKS, rd_chunk = lane % CHUNKS;
       const bool rd_lane = rd_row < ROWS_PER_PASS;
       const int n = n0 + wn * WN + rd_chunk * 8;
+      // this lane's eight columns are the same in every pass: their bias is fetched once
+      uint4 bv = make_uint4(0, 0, 0, 0);
+      if (bias && rd_lane && n < N) bv = *reinterpret_cast<const uint4*>(bias + n);
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -435,7 +455,9 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
           // streaming stores: the tile is not read again by this kernel, and whoever reads
           // it next (the norm kernel) runs on other XCDs; 1 - 3.5 % faster than default stores
           if (rd_lane && r + rd_row < 32 && m < M && n < N) {
-            const u32x4_t v = {lo.x, lo.y, hi.x, hi.y};
+            u32x4_t v = {lo.x, lo.y, hi.x, hi.y};
+            if (bias) v = u32x4_t{add_bias2(lo.x, bv.x), add_bias2(lo.y, bv.y), add_bias2(hi.x, bv.z),
+                                  add_bias2(hi.y, bv.w)};
             __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(out + (size_t)m * ldc + n));
           }
         }
@@ -458,6 +480,11 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
             uint2 v;
             v.x = pack2(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1]);
             v.y = pack2(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+            if (bias) {
+              const uint2 bv = *reinterpret_cast<const uint2*>(bias + n);
+              v.x = add_bias2(v.x, bv.x);
+              v.y = add_bias2(v.y, bv.y);
+            }
             *reinterpret_cast<uint2*>(out + (size_t)m * ldc + n) = v;
           }
         }
@@ -489,7 +516,7 @@ static int launch_big(const GemmBatch& batch, int count, int64_t M, int64_t N, i
   // 16-byte stores need 16-byte aligned row segments that end inside the row
   int wide_store = (N % 8 == 0 && ldc % 8 == 0) ? 1 : 0;
   for (int p = 0; p < count; ++p)
-    if (reinterpret_cast<uintptr_t>(batch.out[p]) & 15u) wide_store = 0;
+    if ((reinterpret_cast<uintptr_t>(batch.out[p]) | reinterpret_cast<uintptr_t>(batch.bias[p])) & 15u) wide_store = 0;
   launch_kernel(gemm_bf16_nt_big_kernel<TM, TN>, dim3((unsigned)grid), dim3(BIG_THREADS), LDS, hs, batch, count,
                 (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n, wide_store);
   return TW_OK;
@@ -554,25 +581,27 @@ static int check_gemm_shape(const char* what, int64_t M, int64_t N, int64_t K, i
   return TW_OK;
 }
 
-static int check_gemm_pointers(const char* what, const void* out, const void* a, const void* b) {
+static int check_gemm_pointers(const char* what, const void* out, const void* a, const void* b,
+                               const void* bias) {
   if (!out || !a || !b) return set_error(TW_ERR_INVALID_ARGUMENT, "%s: null pointer argument", what);
   auto al = [](const void* p, unsigned n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) == 0; };
-  if (!al(a, 16) || !al(b, 16) || !al(out, 8))
-    return set_error(TW_ERR_ALIGNMENT, "%s: needs 16-byte aligned a and b, 8-byte aligned out", what);
+  if (!al(a, 16) || !al(b, 16) || !al(out, 8) || !al(bias, 8))
+    return set_error(TW_ERR_ALIGNMENT, "%s: needs 16-byte aligned a and b, 8-byte aligned out and bias", what);
   return TW_OK;
 }
 
-int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t N, int64_t K,
-                     int64_t ldc, int max_cus, void* stream) {
+int run_gemm_bf16_nt(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N,
+                     int64_t K, int64_t ldc, int max_cus, void* stream) {
   if (int rc = check_gemm_shape("gemm_bf16_nt", M, N, K, ldc)) return rc;
   if (M == 0) return TW_OK;
-  if (int rc = check_gemm_pointers("gemm_bf16_nt", out, a, b)) return rc;
+  if (int rc = check_gemm_pointers("gemm_bf16_nt", out, a, b, bias)) return rc;
   hipStream_t hs = static_cast<hipStream_t>(stream);
   if (big_kernel_fits(M, N, K)) {
     GemmBatch batch = {};
     batch.out[0] = static_cast<uint16_t*>(out);
     batch.a[0] = static_cast<const uint16_t*>(a);
     batch.b[0] = static_cast<const uint16_t*>(b);
+    batch.bias[0] = static_cast<const uint16_t*>(bias);
     if (int rc = launch_big_for(batch, 1, M, N, K, ldc, max_cus, hs)) return rc;
   } else {
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
@@ -581,15 +610,18 @@ int run_gemm_bf16_nt(void* out, const void* a, const void* b, int64_t M, int64_t
     if (grid > INT32_MAX) grid = INT32_MAX;
     launch_kernel(gemm_bf16_nt_kernel, dim3((unsigned)grid), dim3(GEMM_THREADS), 0, hs,
                   static_cast<uint16_t*>(out), static_cast<const uint16_t*>(a),
-                  static_cast<const uint16_t*>(b), (int)M, (int)N, (int)K, ldc, tiles_m, tiles_n);
+                  static_cast<const uint16_t*>(b), static_cast<const uint16_t*>(bias), (int)M, (int)N, (int)K, ldc,
+                  tiles_m, tiles_n);
   }
   return finish_launch("gemm_bf16_nt");
 }
 
-// outs[p][M, N] (row stride ldc) = as[p][M, K] * bs[p][N, K]^T for p < count: one launch
-// over count x tiles when the shape fits the big kernel, one launch per product otherwise.
-int run_gemm_bf16_nt_partials(void* const* outs, const void* const* as, const void* const* bs, int count,
-                              int64_t M, int64_t N, int64_t K, int64_t ldc, int max_cus, void* stream) {
+// outs[p][M, N] (row stride ldc) = as[p][M, K] * bs[p][N, K]^T (+ biases[p] when `biases` and
+// that entry are non-null) for p < count: one launch over count x tiles when the shape fits
+// the big kernel, one launch per product otherwise.
+int run_gemm_bf16_nt_partials(void* const* outs, const void* const* as, const void* const* bs,
+                              const void* const* biases, int count, int64_t M, int64_t N, int64_t K,
+                              int64_t ldc, int max_cus, void* stream) {
   const char* what = "gemm_bf16_nt_partials";
   if (count < 1 || count > TW_MAX_PARTIALS)
     return set_error(TW_ERR_INVALID_ARGUMENT, "%s: number of partials %d not in [1, %d]", what, count,
@@ -599,7 +631,9 @@ int run_gemm_bf16_nt_partials(void* const* outs, const void* const* as, const vo
   if (!outs || !as || !bs) return set_error(TW_ERR_INVALID_ARGUMENT, "%s: null pointer argument", what);
   GemmBatch batch = {};
   for (int p = 0; p < count; ++p) {
-    if (int rc = check_gemm_pointers(what, outs[p], as[p], bs[p])) return rc;
+    const void* bias = biases ? biases[p] : nullptr;
+    if (int rc = check_gemm_pointers(what, outs[p], as[p], bs[p], bias)) return rc;
+    batch.bias[p] = static_cast<const uint16_t*>(bias);
     batch.out[p] = static_cast<uint16_t*>(outs[p]);
     batch.a[p] = static_cast<const uint16_t*>(as[p]);
     batch.b[p] = static_cast<const uint16_t*>(bs[p]);
@@ -609,7 +643,7 @@ int run_gemm_bf16_nt_partials(void* const* outs, const void* const* as, const vo
     return finish_launch(what);
   }
   for (int p = 0; p < count; ++p)
-    if (int rc = run_gemm_bf16_nt(outs[p], as[p], bs[p], M, N, K, ldc, max_cus, stream)) return rc;
+    if (int rc = run_gemm_bf16_nt(outs[p], as[p], bs[p], batch.bias[p], M, N, K, ldc, max_cus, stream)) return rc;
   return TW_OK;
 }
 

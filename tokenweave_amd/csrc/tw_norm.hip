@@ -69,9 +69,10 @@ constexpr int kTraceSlots = 8;
                  (unsigned)__builtin_amdgcn_s_getreg((32 - 1) << 11 | 4)
 #define TW_STAMP_END(row)                                                                        \
   do {                                                                                           \
-    if (threadIdx.x == 0) {                                                                      \
+    unsigned long long* tw_buf = g_trace; /* null outside a traced burst: nothing is written */  \
+    if (threadIdx.x == 0 && tw_buf) {                                                            \
       for (int tw_i = 0; tw_i < kTraceSlots; ++tw_i)                                             \
-        g_trace[(size_t)(row) * kTraceSlots + tw_i] = tw_stamps[tw_i];                           \
+        tw_buf[(size_t)(row) * kTraceSlots + tw_i] = tw_stamps[tw_i];                            \
     }                                                                                            \
   } while (0)
 #else
@@ -571,30 +572,30 @@ __global__ __launch_bounds__(MAXNT) void row_norm_f16_kernel(
 // Split rows: few token rows, many compute units (decode batches).
 //
 // A row is cut into `segs` segments of whole 64-vector chunks and every segment
-// gets its own workgroup, so one row's (P + 1) input streams are pulled by
-// several compute units at once.  A segment workgroup does the first half of the
-// row kernel on its vectors — fp32 sum, rounded residual stored, one sum of
-// squares per chunk by wave_sum — and leaves its chunk sums in the row's slot of
-// a small workspace.  It then counts itself in on the row's arrival counter.  The
-// workgroup that arrives last finds every chunk sum of the row there, reduces
-// them exactly as row_sum_chunks does (chunk c in lane c, one wave_sum), and
-// writes y for the WHOLE row from the rounded residual it re-reads — the same
-// operands in the same order as the one-workgroup kernel, hence the same bits.
-// Nobody waits for anybody: a workgroup that is not last is finished, so the
-// kernel makes progress whatever the dispatch order and needs no co-residency.
+// gets its own workgroup (one vector per lane, one chunk per wave), so one row's
+// (P + 1) input streams are pulled by several compute units at once.  A segment
+// workgroup does the first half of the row kernel on its vectors — fp32 sum,
+// rounded residual stored, one sum of squares per chunk by wave_sum — and leaves
+// its chunk sums in the row's slot of a small workspace.  It then counts itself in
+// on the row's arrival counter.  The workgroup that arrives last finds every chunk
+// sum of the row there, reduces them exactly as row_sum_chunks does (chunk c in
+// lane c, one wave_sum), and writes y for the WHOLE row from the rounded residual
+// it re-reads — the same operands in the same order as the one-workgroup kernel,
+// hence the same bits.  Nobody waits for anybody: a workgroup that is not last is
+// finished, so the kernel makes progress whatever the dispatch order and needs no
+// co-residency.
 //
-// Ordering: what one workgroup hands to another — the rounded residual and the
-// chunk sums — is written with device-scope stores (write-through past the XCD's L2,
-// so no L2 write-back is needed to publish them), every wave waits for its stores to
-// be acknowledged before the workgroup's arrival is counted (a device-scope atomic),
-// and the last workgroup reads them back with device-scope loads, which do not hit
-// in a per-compute-unit cache or another XCD's L2.  The last workgroup of a row
-// resets the row's counter, so the counters are zero again when the kernel ends;
-// calls that share a workspace must not overlap in time.
+// The last workgroup of a row resets the row's counter, so the counters are zero
+// again when the kernel ends; calls that share a workspace must not overlap in time.
 //
-// Workgroup b serves row 8 (b / (8 segs)) + b % 8, segment (b / 8) % segs: the
-// segments of one row have equal b % 8 and so are dispatched to one XCD, whose L2
-// then holds the residual for the last workgroup's re-read.
+// XCD_ROWS: workgroup b serves row 8 (b / (8 segs)) + b % 8, segment (b / 8) % segs,
+// so the segments of one row have equal b % 8 and — with the dispatcher handing
+// consecutive workgroups to consecutive XCDs — run on one XCD, whose L2 then holds
+// the residual for the last workgroup's re-read (0.1 - 0.3 us).  That placement is
+// a speed matter only: the hand-over below is written for segments on different
+// XCDs, and the form without the remap (row = b / segs, segments of a row spread
+// over XCDs) is compiled into the measurement library and checked by the tests
+// against the same bits.
 // ---------------------------------------------------------------------------
 struct SplitRow {
   float sums[kMaxChunks];  // chunk sums of squares of the row in flight (two 128-byte lines)
@@ -612,8 +613,7 @@ __device__ __forceinline__ void store16_device(__amdgpu_buffer_rsrc_t d, uint32_
   __builtin_amdgcn_raw_buffer_store_b128(t, d, off, 0, kStoreDevice);
 }
 
-// XCD_ROWS: the segments of one row are workgroups with equal blockIdx % 8.
-template <int NP, int VPT, bool XCD_ROWS>
+template <int NP, bool XCD_ROWS>
 __global__ __launch_bounds__(1024) void row_norm_split_kernel(
     PartialPtrs parts, int np_rt, void* y_out, void* residual, const void* __restrict__ weight,
     SplitRow* __restrict__ ws, float eps, int num_tokens, int vec_per_row, float hidden, int segs, int nt) {
@@ -633,69 +633,65 @@ __global__ __launch_bounds__(1024) void row_norm_split_kernel(
   // that follow find their cache lines there.
   asm volatile("" ::"s"(parts.p[0]));
   if (row >= num_tokens) return;
-  const int chunk0 = seg * VPT * nwaves;  // first chunk of this segment
-
-  uint32_t off[VPT];
-#pragma unroll
-  for (int k = 0; k < VPT; ++k) off[k] = (uint32_t)((chunk0 + k * nwaves) * 64 + (int)threadIdx.x) * 16u;
+  const int chunk = seg * nwaves + wave;  // this wave's chunk of the row
+  const uint32_t off = (uint32_t)(chunk * 64 + lane) * 16u;
 
   const __amdgpu_buffer_rsrc_t dr = row_desc(residual, row, row_bytes);
-  float s[VPT][8];
+  float s[8];
   if (NP > 0) {
-    uint4 a[VPT][NP > 0 ? NP : 1];
-    uint4 rv[VPT];
+    uint4 a[NP > 0 ? NP : 1];
 #pragma unroll
-    for (int p = 0; p < NP; ++p) {
-      const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[p], row, row_bytes);
+    for (int p = 0; p < NP; ++p) a[p] = load16<kLoadStream>(row_desc(parts.p[p], row, row_bytes), off);
+    const uint4 rv = load16<kLoadStream>(dr, off);
+    unpack8(a[0], s);
 #pragma unroll
-      for (int k = 0; k < VPT; ++k) a[k][p] = load16<kLoadStream>(dp, off[k]);
-    }
-#pragma unroll
-    for (int k = 0; k < VPT; ++k) rv[k] = load16<kLoadStream>(dr, off[k]);
-#pragma unroll
-    for (int k = 0; k < VPT; ++k) unpack8(a[k][0], s[k]);
-#pragma unroll
-    for (int p = 1; p < NP; ++p) {
-#pragma unroll
-      for (int k = 0; k < VPT; ++k) add8(a[k][p], s[k]);
-    }
-#pragma unroll
-    for (int k = 0; k < VPT; ++k) add8(rv[k], s[k]);
+    for (int p = 1; p < NP; ++p) add8(a[p], s);
+    add8(rv, s);
   } else {
-    {
-      const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[0], row, row_bytes);
-#pragma unroll
-      for (int k = 0; k < VPT; ++k) unpack8(load16<kLoadStream>(dp, off[k]), s[k]);
-    }
-    for (int p = 1; p < np; ++p) {
-      const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[p], row, row_bytes);
-#pragma unroll
-      for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dp, off[k]), s[k]);
-    }
-#pragma unroll
-    for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dr, off[k]), s[k]);
+    unpack8(load16<kLoadStream>(row_desc(parts.p[0], row, row_bytes), off), s);
+    for (int p = 1; p < np; ++p) add8(load16<kLoadStream>(row_desc(parts.p[p], row, row_bytes), off), s);
+    add8(load16<kLoadStream>(dr, off), s);
   }
 
   SplitRow* slot = ws + row;
-#pragma unroll
-  for (int k = 0; k < VPT; ++k) {
+  {
     float ss = 0.0f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) ss += s[k][e] * s[k][e];
+    for (int e = 0; e < 8; ++e) ss += s[e] * s[e];
     uint4 rnew;
-    rnew.x = pack_bf16(s[k][0], s[k][1]);
-    rnew.y = pack_bf16(s[k][2], s[k][3]);
-    rnew.z = pack_bf16(s[k][4], s[k][5]);
-    rnew.w = pack_bf16(s[k][6], s[k][7]);
-    store16_device(dr, off[k], rnew);
+    rnew.x = pack_bf16(s[0], s[1]);
+    rnew.y = pack_bf16(s[2], s[3]);
+    rnew.z = pack_bf16(s[4], s[5]);
+    rnew.w = pack_bf16(s[6], s[7]);
+    store16_device(dr, off, rnew);
     const float c = wave_sum(ss);
-    const int chunk = chunk0 + k * nwaves + wave;
     if (lane == 0 && chunk < nchunks)
       __hip_atomic_store(&slot->sums[chunk], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
-  // every store of this wave has been acknowledged at device scope before the
-  // workgroup's arrival is counted
+  // The hand-over, instruction by instruction.  It is built from device-scope accesses
+  // and explicit waits instead of release / acquire fences, because a fence at agent
+  // scope is an L2 write-back (buffer_wbl2) per wave, serialised per XCD: 2 - 20x the
+  // kernel's whole duration.  What it relies on is stated here so that it can be checked:
+  //  (1) Everything another workgroup will read — the rounded residual (store16_device)
+  //      and the chunk sums (relaxed agent-scope atomic stores) — is written with sc1
+  //      stores: the data is written through this XCD's L2 to memory, and the store's
+  //      acknowledgement (what vmcnt counts) comes back only after that.  No dirty line
+  //      is left behind in an L2 that another XCD cannot see, so nothing needs writing back.
+  //  (2) s_waitcnt vmcnt(0): this wave goes on only when every one of its stores has
+  //      been acknowledged.  s_barrier: every wave of the workgroup has done so.
+  //  (3) Only then thread 0 counts the workgroup in, with an agent-scope atomic
+  //      read-modify-write (performed at the memory side, one total order per counter).
+  //      A workgroup that reads segs - 1 therefore knows that every other segment's
+  //      stores of (1) were acknowledged before that segment's increment, which precedes
+  //      its own in the counter's order.
+  //  (4) The last workgroup's reads of the chunk sums and of the residual are issued after
+  //      the atomic's value has come back (the branch below depends on it; vector memory
+  //      instructions are issued in program order, never speculatively), and they are sc1
+  //      loads: served from memory at device scope, not from a line an earlier access may
+  //      have left in this compute unit's cache or this XCD's L2.  The residual lines are
+  //      read before that only by the segment that overwrites them, with streaming loads.
+  //  The weight row and y are ordinary traffic: nobody else reads or writes them here.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (threadIdx.x == 0)
@@ -965,8 +961,8 @@ static bool splittable(bool vec_ok, int dtype, const void* residual, const void*
 
 // Segments per row and workgroup shape of the split-row kernel, or false when the
 // one-workgroup-per-row kernel is the better (or only) choice.  A segment is
-// vpt * nwaves whole chunks.
-struct SplitPlan { int vpt, nwaves, segs; };
+// nwaves whole chunks, one per wave.
+struct SplitPlan { int nwaves, segs; };
 
 static bool split_plan(int V, int64_t T, int cus, SplitPlan* sp) {
   const int nchunks = (V + 63) / 64;
@@ -979,7 +975,6 @@ static bool split_plan(int V, int64_t T, int cus, SplitPlan* sp) {
   // hand-over costs more than the shorter load phase saves).  Eight-chunk segments take
   // over when four-chunk ones would make more workgroups than there are compute units.
   if (T > 48 || nchunks < 16) return false;
-  sp->vpt = 1;
   sp->nwaves = T * ((nchunks + 3) / 4) <= cus ? 4 : 8;
   sp->segs = (nchunks + sp->nwaves - 1) / sp->nwaves;
   return sp->segs >= 2;
@@ -990,13 +985,8 @@ static void launch_split(const RowNormArgs& a, const SplitPlan& sp) {
   const int V = (int)(a.H / 8);
   const int groups = (int)((a.T + 7) / 8);
   dim3 g((unsigned)(groups * 8 * sp.segs)), b((unsigned)(sp.nwaves * 64));
-#define TW_LAUNCH_SPLIT(VPT)                                                                     \
-  launch_kernel(row_norm_split_kernel<NP, VPT, true>, g, b, 0, a.stream, a.parts, a.np, a.y,     \
-                a.residual, a.weight, a.split_ws, a.eps, (int)a.T, V, (float)a.H, sp.segs, sp.nwaves * 64)
-  if (sp.vpt == 1) TW_LAUNCH_SPLIT(1);
-  else if (sp.vpt == 2) TW_LAUNCH_SPLIT(2);
-  else TW_LAUNCH_SPLIT(4);
-#undef TW_LAUNCH_SPLIT
+  launch_kernel(row_norm_split_kernel<NP, true>, g, b, 0, a.stream, a.parts, a.np, a.y, a.residual, a.weight,
+                a.split_ws, a.eps, (int)a.T, V, (float)a.H, sp.segs, sp.nwaves * 64);
 }
 
 static void launch_split_np(const RowNormArgs& a, const SplitPlan& sp) {

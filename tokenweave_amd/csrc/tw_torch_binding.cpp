@@ -11,6 +11,7 @@
 #include <ATen/ATen.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <hip/hip_runtime_api.h>
 #include <torch/library.h>
 
 #include <map>
@@ -142,21 +143,44 @@ int64_t peer_stride(uint64_t mcptr, int64_t world_size, int64_t nbytes) {
 
 // ---------------------------------------------------------------------------
 // Workspace of the split-row kernel: one zeroed buffer per (device, stream), made on
-// the first decode-size call on that stream and kept for the life of the process.
+// the first decode-size call on that stream — never while the stream is being captured
+// into a graph — and kept for the life of the process.
 // ---------------------------------------------------------------------------
 std::mutex g_ws_mutex;
 std::unordered_map<uint64_t, Tensor> g_workspaces;
 
-void* split_workspace(const Tensor& like, void* stream) {
-  const uint64_t key = ((uint64_t)(uintptr_t)stream << 8) ^ (uint64_t)(like.device().index() & 0xff);
+bool stream_is_capturing(void* stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  // a failing query leaves the capture (if any) alone; treat it as "capturing": do not allocate
+  if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &status) != hipSuccess) return true;
+  return status != hipStreamCaptureStatusNone;
+}
+
+// The workspace of (device, stream), or null when there is none yet and the stream is
+// being captured: allocating then would draw from the graph's private pool and record the
+// fill kernel.  The caller runs the one-workgroup-per-row kernel instead (same bits); a
+// workspace made beforehand (prepare_split_workspace or any eager decode-size call on the
+// stream) is used by captured calls too.
+void* split_workspace(const c10::Device& device, void* stream) {
+  const uint64_t key = ((uint64_t)(uintptr_t)stream << 8) ^ (uint64_t)(device.index() & 0xff);
   std::lock_guard<std::mutex> lock(g_ws_mutex);
   auto it = g_workspaces.find(key);
   if (it == g_workspaces.end()) {
-    Tensor ws = at::zeros({(int64_t)TW_SPLIT_WORKSPACE_BYTES}, like.options().dtype(at::kByte));
+    if (stream_is_capturing(stream)) return nullptr;
+    Tensor ws = at::zeros({(int64_t)TW_SPLIT_WORKSPACE_BYTES}, at::TensorOptions().device(device).dtype(at::kByte));
     TORCH_CHECK(((uintptr_t)ws.data_ptr() & 255u) == 0, "workspace allocation is not 256-byte aligned");
     it = g_workspaces.emplace(key, std::move(ws)).first;
   }
   return it->second.data_ptr();
+}
+
+// Creates the workspace of the current stream of device `device_index` now (before a capture).
+void prepare_split_workspace(int64_t device_index) {
+  const c10::Device device(c10::DeviceType::CUDA, (c10::DeviceIndex)device_index);
+  c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device);
+  void* stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device.index()).stream();
+  TORCH_CHECK(split_workspace(device, stream) != nullptr,
+              "prepare_split_workspace: the current stream is being captured; call it before the capture begins");
 }
 
 // ---------------------------------------------------------------------------
@@ -231,10 +255,12 @@ void fused_rs_ln(bool all_gather, const char* kernel, Tensor& input, Tensor& res
   Launch l(input);
   if (max_ctas <= 0 && r.T > 0 && r.T <= TW_SPLIT_MAX_TOKENS) {
     // decode-size batch: several workgroups per row where that pays
-    check_rc(tw_fused_rs_ln_ag_cta_ws(input.data_ptr(), residual.data_ptr(), weight.data_ptr(), (uint64_t)mcptr,
-                                      stride, (int)rank, (int)world_size, 0, (float)epsilon, r.T, r.H,
-                                      split_workspace(input, l.stream), TW_SPLIT_WORKSPACE_BYTES, l.stream));
-    return;
+    if (void* ws = split_workspace(dev, l.stream)) {
+      check_rc(tw_fused_rs_ln_ag_cta_ws(input.data_ptr(), residual.data_ptr(), weight.data_ptr(), (uint64_t)mcptr,
+                                        stride, (int)rank, (int)world_size, 0, (float)epsilon, r.T, r.H, ws,
+                                        TW_SPLIT_WORKSPACE_BYTES, l.stream));
+      return;
+    }
   }
   auto fn = all_gather ? tw_fused_rs_ln_ag_cta : tw_fused_rs_ln_cta;
   check_rc(fn(input.data_ptr(), residual.data_ptr(), weight.data_ptr(), (uint64_t)mcptr, stride, (int)rank,
@@ -371,6 +397,8 @@ TORCH_LIBRARY(tokenweave_amd, m) {
   m.def("register_partials_region(int base, int stride_bytes, int slots, int usable_bytes, int token) -> ()",
         &register_partials_region);
   m.def("unregister_partials_region(int base, int token) -> ()", &unregister_partials_region);
+  // the split-row workspace of the current stream, ahead of a graph capture
+  m.def("prepare_split_workspace(int device_index) -> ()", &prepare_split_workspace);
 }
 
 TORCH_LIBRARY_IMPL(tokenweave_amd, CUDA, m) {

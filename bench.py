@@ -74,6 +74,8 @@ def bench_lib():
         L.twb_trace_stream_rows.argtypes = [ctypes.POINTER(vp), vp, i64, i64, vp]
         L.twb_empty.argtypes = [ci, ci, vp]
         L.twb_clock_probe.argtypes = [vp, ci, vp]
+        L.twb_touch_pages.argtypes = [vp, i64, vp, i64, ci, ci, vp, vp]
+        L.twb_latency_chain.argtypes = [vp, i64, ci, i64, vp, vp, vp]
         L.twb_trace_reduce_add_rms_norm.argtypes = [ctypes.POINTER(vp), ci, vp, vp, vp, i64, i64, ci, f32, vp, vp]
         L.twb_gemm_loop.argtypes = [ci, ci, i64, vp, vp, vp, ci, vp]
         L.twb_lds_read_rate.argtypes = [ci, ci, ci, vp, vp, vp, ci, vp]
@@ -102,6 +104,9 @@ def parse_args():
     ap.add_argument("--gemm-limits", action="store_true",
                     help="time the GEMM's k loop assembled from its parts (MFMAs, LDS fragment reads, operand "
                          "slabs global -> LDS) on L2-resident operands, and the LDS read rate, and print them")
+    ap.add_argument("--gemm-scaling", action="store_true",
+                    help="time the big GEMM kernel's 320 x 256 tile, one tile per compute unit, on 32 .. 256 "
+                         "compute units (K = 1024 and 8192) with the shader clock rocm-smi reports meanwhile")
     ap.add_argument("--weave-only", action="store_true",
                     help="time only the GEMM + norm weave of config 5 and print its figures (for profiling)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -115,6 +120,16 @@ def parse_args():
     ap.add_argument("--timeline", action="store_true",
                     help="run the workload through the stamped build of the norm kernel and print the "
                          "per-workgroup timeline breakdown")
+    ap.add_argument("--pretouch", type=int, default=0, metavar="STEP_BYTES",
+                    help="before every launch, an untimed-by-itself helper kernel reads one dword per STEP_BYTES "
+                         "of the launch's inputs from every XCD (address translations warm, data still cold); "
+                         "for counter runs")
+    ap.add_argument("--graph-replay", action="store_true",
+                    help="time the workload under HIP-graph replay (two passes over the rotating input sets in "
+                         "one graph) and print microseconds per launch")
+    ap.add_argument("--tlb-latency", action="store_true",
+                    help="measure the latency of dependent cold reads with and without a cached address "
+                         "translation and print it")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline")
     return ap.parse_args()
 
@@ -124,15 +139,19 @@ class NormRunner:
     ctypes call per launch) for each input set, so that the host enqueues a step
     faster than the GPU runs it."""
 
-    def __init__(self, cfg, nsets, max_ctas, device, epilogue="bf16", split=None):
+    def __init__(self, cfg, nsets, max_ctas, device, epilogue="bf16", split=None, pretouch=0):
         import torch
         from tokenweave_amd import _custom_ops as ops
         from tokenweave_amd import _lib
         from tokenweave_amd import workloads as wl
         self.calls = []
+        self.inputs = []
+        self.pretouch = pretouch
+        self.sink = torch.zeros(256, dtype=torch.uint8, device=device) if pretouch else None
         L = _lib.lib()
         for i in range(nsets):
             inp = wl.make_norm_inputs(cfg, device, seed_offset=i)
+            self.inputs.append(inp)
             if epilogue == "bf16":
                 # y lands on this rank's staging rows (rank 0)
                 op = ops.bind_reduce_add_rms_norm(inp.partials, inp.partials[0], inp.residual, inp.weight,
@@ -166,7 +185,17 @@ class NormRunner:
                 1 if epilogue == "int8_dynamic" else 0)
         return ops.BoundOp(L.tw_reduce_add_rms_norm_dynamic_per_token_quant, args, keep, out.device)
 
+    def touch(self, i, stream, step_bytes):
+        """Page-touch the inputs of step i: one dword per `step_bytes` of the P partial
+        buffers and of the residual, read from every XCD."""
+        inp = self.inputs[i % len(self.inputs)]
+        st, r = inp.staging, inp.residual
+        bench_check(bench_lib().twb_touch_pages(st.data_ptr(), st.numel() * 2, r.data_ptr(), r.numel() * 2,
+                                                step_bytes, 4, self.sink.data_ptr(), stream.cuda_stream))
+
     def step(self, i, stream):
+        if self.pretouch:
+            self.touch(i, stream, self.pretouch)
         self.calls[i % len(self.calls)](stream)
 
 
@@ -184,7 +213,7 @@ LEAD_IN = 40        # untimed launches ahead of an event bracket (the bracket st
 
 
 def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16", regions=REGIONS, preroll_ms=PREROLL_MS,
-              lead_in=LEAD_IN, split=None):
+              lead_in=LEAD_IN, split=None, pretouch=0):
     """After an untimed pre-roll and `warmup` warm-up launches, times `regions` regions of
     exactly `steps` back-to-back launches twice over: by the wall clock between two device
     synchronisations (ms_per_step, gbps), and by HIP events on the launch stream around
@@ -195,7 +224,7 @@ def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16", regions=REG
     free, _ = torch.cuda.mem_get_info()
     set_bytes = (cfg.P + 1) * cfg.T * cfg.H * 2 + cfg.H * 2
     nsets = max(2, min(nsets, int(free * 0.6) // (set_bytes * 3)))  # fp32 staging while generating
-    runner = NormRunner(cfg, nsets, max_ctas, device, epilogue, split)
+    runner = NormRunner(cfg, nsets, max_ctas, device, epilogue, split, pretouch)
     stream = torch.cuda.current_stream()
     it = 0
     preroll_steps = max(warmup, int(preroll_ms * 1e3 / max(2.0, cfg.bytes / 6e6)))
@@ -242,6 +271,85 @@ def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16", regions=REG
     del runner
     torch.cuda.empty_cache()
     return res
+
+
+def time_tlb_latency(device):
+    """What an address-translation miss costs a cold read.  One lane reads dwords one after
+    the other (each waits for the one before) from two 4 GiB regions A and B, always from
+    cache lines that nothing has read since they were written (cold data):
+      pass 1  A, one read per 2 MiB                      (translations as the fill left them)
+      pass 2  B likewise                                 (pushes A's translations out of any TLB
+                                                          that cannot hold 2 x 2048 of them)
+      pass 3  A again, other lines of the same pages     (warm only if the TLBs reach > 8 GiB)
+      pass 4  A again, other lines, right after pass 3   (translations warm, data cold)
+      pass 5  A, 32 reads per 64 KiB inside 2 MiB pages  (same page back to back: the floor)
+    Microseconds per read: median and 90th percentile."""
+    import numpy as np
+    import torch
+    L = bench_lib()
+    sp = torch.cuda.current_stream().cuda_stream
+    size = 4 << 30
+    A = torch.empty(size, dtype=torch.uint8, device=device)
+    B = torch.empty(size, dtype=torch.uint8, device=device)
+    A.random_(0, 200)
+    B.random_(0, 200)
+    torch.cuda.synchronize()
+    n = size // (2 << 20)
+    out = torch.zeros(n * 4, dtype=torch.int32, device=device)
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+
+    def chain(buf, stride, count, offset):
+        bench_check(L.twb_latency_chain(buf.data_ptr(), stride, count, offset, out.data_ptr(), sink.data_ptr(), sp))
+        torch.cuda.synchronize()
+        t = out[:count].cpu().numpy().astype(np.float64) * 0.01
+        return {"reads": count, "median_us": round(float(np.median(t)), 3), "p10_us": round(float(np.percentile(t, 10)), 3),
+                "p90_us": round(float(np.percentile(t, 90)), 3)}
+
+    res = {"region_bytes": size, "page_stride_bytes": 2 << 20}
+    res["pass1_A_first_touch"] = chain(A, 2 << 20, n, 0)
+    res["pass2_B_first_touch"] = chain(B, 2 << 20, n, 0)
+    res["pass3_A_after_B_other_lines"] = chain(A, 2 << 20, n, 8192)
+    res["pass4_A_again_other_lines"] = chain(A, 2 << 20, n, 16384)
+    res["pass5_A_64KiB_steps_inside_pages"] = chain(A, 64 << 10, 4096, 32768)
+    res["pass6_A_first_256_pages_again"] = chain(A, 2 << 20, 256, 24576)
+    res["pass7_A_first_256_pages_again"] = chain(A, 2 << 20, 256, 28672)
+    for k, v in res.items():
+        log(f"[tlb-latency] {k}: {v}")
+    return res
+
+
+def time_graph_replay(cfg, max_ctas, device, cycles=2, replays=5, brackets=7):
+    """The workload under HIP-graph replay: `cycles` passes over the rotating input sets
+    (4 GiB, cold data) captured into one graph, timed per launch by HIP events around
+    `replays` replays (median of `brackets`): the launches back to back with no host in the
+    loop — what is left of the launch-to-launch gap when the host is out of the picture."""
+    import torch
+    nsets = max(2, min(256, -(-ROTATION_BYTES // cfg.bytes)))
+    runner = NormRunner(cfg, nsets, max_ctas, device)
+    main_s, _ = weave_streams()
+    launches = cycles * nsets
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=main_s):
+        for i in range(launches):
+            runner.step(i, main_s)
+    ts = []
+    with torch.cuda.stream(main_s):
+        g.replay()
+        torch.cuda.synchronize()
+        for _ in range(brackets):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(main_s)
+            for _ in range(replays):
+                g.replay()
+            e1.record(main_s)
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3 / (replays * launches))
+    out = {"workload": cfg.name, "launches_per_graph": launches, "rotating_input_sets": nsets,
+           "replays_per_bracket": replays, "brackets": brackets,
+           "us_per_launch": round(statistics.median(ts), 3), "min": round(min(ts), 3), "max": round(max(ts), 3)}
+    del g, runner
+    torch.cuda.empty_cache()
+    return out
 
 
 CALIBRATION_COPY_BYTES = 256 << 20
@@ -831,9 +939,83 @@ def time_gemm_limits(device):
             "loop": loop, "lds_read_rate": lds}
 
 
+def time_gemm_scaling(device, seconds=2.0):
+    """How the big GEMM kernel's speed per compute unit depends on how many compute units run it.
+    [320 c / 32, K] x [8192, K]^T with the grid capped at c workgroups is c tiles of 320 x 256, one per
+    compute unit, a single round — the same work per compute unit for every c.  Each point runs for
+    `seconds` of back-to-back launches (HIP events, median) while a thread samples `rocm-smi
+    --showclocks`; sclk is the median shader clock it reported.  Per compute unit the nominal peak is
+    2500 / 256 = 9.77 TFLOP/s at 2.4 GHz."""
+    import re
+    import subprocess
+    import threading
+    import torch
+    from tokenweave_amd import _custom_ops as ops
+    from tokenweave_amd import workloads as wl
+    stream = torch.cuda.current_stream()
+
+    def sclk_mhz():
+        try:
+            txt = subprocess.run(["rocm-smi", "--showclocks", "--json"], capture_output=True, text=True,
+                                 timeout=10).stdout
+            card = json.loads(txt)
+            card = card[sorted(card)[0]]
+            for k, v in card.items():
+                if k.startswith("sclk clock speed"):
+                    m = re.search(r"([0-9.]+)", str(v))
+                    return float(m.group(1)) if m else None
+        except Exception:   # no rocm-smi, no permission, other output: the clock column stays empty
+            return None
+        return None
+
+    out = {"definitions": "one 320 x 256 tile per compute unit on `cus` compute units (grid cap), N = 8192; "
+                          "tflops_per_cu against a nominal 9.77; sclk_mhz = median of rocm-smi samples during the run"}
+    for K in (1024, 8192):
+        rows = []
+        for cus in (32, 64, 128, 192, 224, 256):
+            M = 320 * cus // 32
+            g = wl.make_gemm_inputs(M, 8192, K, device)
+            outs = [torch.zeros((M, 8192), dtype=torch.bfloat16, device=device) for _ in range(4)]
+            calls = [ops.bind_gemm_bf16_nt(o, g.a, g.b, cus) for o in outs]
+            for i in range(20):
+                calls[i % 4](stream)
+            torch.cuda.synchronize()
+            samples, stop = [], threading.Event()
+
+            def sampler():
+                while not stop.is_set():
+                    samples.append(sclk_mhz())
+                    time.sleep(0.05)
+            th = threading.Thread(target=sampler)
+            th.start()
+            ts, t_end = [], time.perf_counter() + seconds
+            while time.perf_counter() < t_end:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for i in range(200):
+                    calls[i % 4](stream)
+                e1.record(stream)
+                torch.cuda.synchronize()
+                ts.append(e0.elapsed_time(e1) * 1e3 / 200)
+            stop.set()
+            th.join()
+            us = statistics.median(ts)
+            tf = 2.0 * M * 8192 * K / us / 1e6
+            clk = [c for c in samples[2:] if c]
+            rows.append({"cus": cus, "M": M, "us": round(us, 2), "tflops": round(tf, 1),
+                         "tflops_per_cu": round(tf / cus, 2),
+                         "share_of_nominal_per_cu": round(tf / cus / (MFMA_BF16_PEAK_TFLOPS / 256), 3),
+                         "sclk_mhz": round(statistics.median(clk)) if clk else None})
+            log(f"[gemm-scaling] K={K}: {rows[-1]}")
+            del outs, calls, g
+            torch.cuda.empty_cache()
+        out[f"K{K}"] = rows
+    return out
+
+
 def weave_block(device, steps):
     """Both forms of config 5 for the JSON line."""
-    caps = (128, 160, 192, 224, 240)
+    caps = (128, 160, 176, 192, 208, 224, 240)
     return {"workload": "c5 token weave: GEMM [2458, 1024] x [8192, 1024]^T of one split || fused P=8 norm of "
                         "the 1638-row split, H=8192",
             "definitions": "serial = both kernels on one stream; overlap = GEMM capped to gemm_cus compute "
@@ -867,6 +1049,12 @@ def main():
     if args.host_cost:
         print(json.dumps({"host_us_per_call": host_cost(device)}), flush=True)
         return
+    if args.tlb_latency:
+        print(json.dumps({"tlb_latency": time_tlb_latency(device)}), flush=True)
+        return
+    if args.graph_replay:
+        print(json.dumps({"graph_replay": time_graph_replay(cfg, args.max_ctas, device)}), flush=True)
+        return
     if args.timeline:
         print(json.dumps({"timeline": time_timeline(cfg, device), "arrivals": time_arrivals(cfg, device)}),
               flush=True)
@@ -877,13 +1065,16 @@ def main():
     if args.gemm_limits:
         print(json.dumps({"gemm_limits": time_gemm_limits(device)}), flush=True)
         return
+    if args.gemm_scaling:
+        print(json.dumps({"gemm_scaling": time_gemm_scaling(device)}), flush=True)
+        return
     if args.weave_only:
         print(json.dumps({"weave": weave_block(device, 20)}), flush=True)
         return
     log(f"[bench] {torch.cuda.get_device_name(0)}; workload {cfg.name}: P={cfg.P} T={cfg.T} "
         f"H={cfg.H} bytes/call={cfg.bytes}")
 
-    res = time_norm(cfg, args.steps, args.warmup, args.max_ctas, device)
+    res = time_norm(cfg, args.steps, args.warmup, args.max_ctas, device, pretouch=args.pretouch)
     log(f"[bench] {res}")
     kernel_us = res["event_us_per_launch"]
     traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name, (None, None)) if args.max_ctas == 0 else (None, None)

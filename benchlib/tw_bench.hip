@@ -160,6 +160,42 @@ __global__ __launch_bounds__(256) void copy16_kernel(uint4* __restrict__ dst, co
 
 __global__ void empty_kernel() {}
 
+// Reads one dword every `step` bytes of two regions, from every XCD (workgroup b runs on
+// XCD b % 8 and takes the addresses of slice b / 8): afterwards the address translations
+// of the regions are in the translation caches of every XCD while (with step >= 4 KiB)
+// next to none of their data is in any cache.  Streaming loads, nothing written unless the
+// data matches a pattern that random inputs never produce.
+__global__ __launch_bounds__(64) void touch_pages_kernel(const uint8_t* a, uint64_t a_bytes, const uint8_t* b,
+                                                         uint64_t b_bytes, uint32_t step, uint32_t* sink) {
+  const uint64_t slices = gridDim.x >> 3, slice = blockIdx.x >> 3;
+  uint32_t v = 0;
+  for (uint64_t off = (slice * 64 + threadIdx.x) * (uint64_t)step; off < a_bytes; off += slices * 64 * step)
+    v ^= __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(a + off));
+  for (uint64_t off = (slice * 64 + threadIdx.x) * (uint64_t)step; off < b_bytes; off += slices * 64 * step)
+    v ^= __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(b + off));
+  if (v == 0x5eed5eedu) sink[threadIdx.x] = v;
+}
+
+// One lane reads `count` dwords, `stride` bytes apart from base + offset, one after the
+// other (each read waits for the previous one), and notes how long each took on the
+// constant-rate wall clock (10 ns units): out[k] = latency of read k.  Streaming loads:
+// nothing is kept in a cache on the way.
+__global__ __launch_bounds__(64) void latency_chain_kernel(const uint8_t* base, uint64_t stride, int count,
+                                                           uint64_t offset, uint32_t* out, uint32_t* sink) {
+  if (threadIdx.x != 0) return;
+  uint32_t acc = 0;
+  for (int k = 0; k < count; ++k) {
+    const uint32_t* p = reinterpret_cast<const uint32_t*>(base + (uint64_t)k * stride + offset);
+    const unsigned long long t0 = wall_clock64();
+    const uint32_t v = __builtin_nontemporal_load(p);
+    asm volatile("s_waitcnt vmcnt(0)" ::"v"(v) : "memory");
+    const unsigned long long t1 = wall_clock64();
+    acc ^= v;
+    out[k] = (uint32_t)(t1 - t0);
+  }
+  if (acc == 0x5eed5eedu) sink[0] = acc;
+}
+
 // One wave that watches both clocks for `ticks` units of the constant-rate wall clock
 // (10 ns each): out[0] = shader-clock cycles, out[1] = wall-clock ticks that went by.  The
 // ratio is the shader clock the compute unit ran at during the window.
@@ -380,6 +416,34 @@ TWB_API int twb_empty(int grid, int block, void* stream) {
   tw::launch_kernel(twb::empty_kernel, dim3((unsigned)grid), dim3((unsigned)block), 0,
                     static_cast<hipStream_t>(stream));
   return tw::finish_launch("empty");
+}
+
+// See touch_pages_kernel.  a, b: device regions (b may be null), sizes in bytes; step: a
+// multiple of 4, at least 128; sink: 256 bytes of device memory; grid = 8 * slices workgroups.
+TWB_API int twb_touch_pages(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes, int step, int slices,
+                            void* sink, void* stream) {
+  if (!a || a_bytes < 4 || (b && b_bytes < 4) || step < 128 || step % 4 != 0 || slices < 1 || slices > 4096 ||
+      !sink || (reinterpret_cast<uintptr_t>(a) & 3u) || (reinterpret_cast<uintptr_t>(b) & 3u))
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "touch_pages: bad argument");
+  // the last dword read of a region starts at a multiple of step below bytes - 3
+  tw::launch_kernel(twb::touch_pages_kernel, dim3((unsigned)(8 * slices)), dim3(64), 0,
+                    static_cast<hipStream_t>(stream), static_cast<const uint8_t*>(a), (uint64_t)(a_bytes - 3),
+                    static_cast<const uint8_t*>(b), (uint64_t)(b ? b_bytes - 3 : 0), (uint32_t)step,
+                    static_cast<uint32_t*>(sink));
+  return tw::finish_launch("touch_pages");
+}
+
+// See latency_chain_kernel.  base: device region of at least (count - 1) * stride + offset + 4
+// bytes; out: count uint32 of device memory; sink: 4 bytes.
+TWB_API int twb_latency_chain(const void* base, int64_t stride, int count, int64_t offset, void* out, void* sink,
+                              void* stream) {
+  if (!base || !out || !sink || stride < 4 || stride % 4 != 0 || offset < 0 || offset % 4 != 0 || count < 1 ||
+      count > (1 << 20) || (reinterpret_cast<uintptr_t>(base) & 3u))
+    return tw::set_error(TW_ERR_INVALID_ARGUMENT, "latency_chain: bad argument");
+  tw::launch_kernel(twb::latency_chain_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                    static_cast<const uint8_t*>(base), (uint64_t)stride, count, (uint64_t)offset,
+                    static_cast<uint32_t*>(out), static_cast<uint32_t*>(sink));
+  return tw::finish_launch("latency_chain");
 }
 
 // Shader clock over a window of `microseconds` (1 .. 1000) on one compute unit: out is two

@@ -142,7 +142,8 @@ TW_API int tw_fused_rs_ln_ag_cta(void* input, void* residual, const void* weight
  * 256-byte aligned, all zeros before the first call that uses it.  Every call
  * leaves it ready for the next one (its arrival counters back at zero) when its
  * kernel has finished.  Calls that share a workspace must not overlap in time
- * (same stream, or ordered by events). */
+ * (same stream, or ordered by events).  It holds the hand-over slots of
+ * TW_SPLIT_MAX_TOKENS rows that are cut into segments. */
 #define TW_SPLIT_MAX_TOKENS 256
 #define TW_SPLIT_WORKSPACE_BYTES (TW_SPLIT_MAX_TOKENS * 384)
 
@@ -152,8 +153,13 @@ TW_API int tw_fused_rs_ln_ag_cta(void* input, void* residual, const void* weight
  * `workspace`, and the workgroup that arrives last normalises the row.  Results
  * are bit-identical to tw_reduce_add_rms_norm.  The split is used when
  * max_ctas <= 0, num_tokens <= TW_SPLIT_MAX_TOKENS and tw_split_segments() says
- * more than one segment; otherwise, or with workspace == NULL, the call IS
- * tw_reduce_add_rms_norm.  workspace_bytes < TW_SPLIT_WORKSPACE_BYTES is an error.
+ * more than one segment.  The workspace also serves batches of a few more rows
+ * than the device has compute units (C < num_tokens <= C + C/4): one workgroup
+ * per row would give some units two rows and the others one, so the first C rows
+ * get a workgroup each and the excess rows are cut into quarters, a workgroup
+ * each, handed over the same way (bit-identical again).  Otherwise, or
+ * with workspace == NULL, the call IS tw_reduce_add_rms_norm.
+ * workspace_bytes < TW_SPLIT_WORKSPACE_BYTES is an error.
  * The reference sizes its persistent grids per batch so that its kernels are not
  * starved of CTAs (grid = min(MAX_CTAS, rows), block = hidden_size / 8:
  * csrc/tokenweave_fused_kernels.cu:241-244, vllm/model_executor/models/
@@ -193,7 +199,8 @@ TW_API int tw_reduce_add_rms_norm_noalloc(const void* const* partials, int num_p
                                    int max_ctas, float epsilon, void* stream);
 
 /* Segments per row the *_ws entry points use for this shape on the current
- * device: 1 = one workgroup per row (no workspace traffic). */
+ * device: 1 = one workgroup per row (no workspace traffic).  For a batch of a few
+ * more rows than compute units it is the number of segments of each excess row. */
 TW_API int tw_split_segments(int64_t num_tokens, int64_t hidden_size, int max_ctas);
 
 /* out[M, N] = a[M, K] * b[N, K]^T, bf16 in, fp32 accumulate on MFMA, bf16 out.

@@ -227,6 +227,43 @@ def test_soak_alternating_decode_shapes_on_one_workspace(form, launches):
     assert int(ws.view(torch.int32).view(-1, 96)[:, 64].abs().max()) == 0, "an arrival counter was left non-zero"
 
 
+# ---------------------------------------------------------------------------
+# mixed launch: a few more rows than compute units
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("H", [8192, 6144, 4608, 2048])
+@pytest.mark.parametrize("P", [1, 8, 3])
+@pytest.mark.parametrize("extra", [1, 8, 13, 32, 47, 64])
+def test_mixed_launch_bit_identical(extra, P, H):
+    """C + extra rows (extra <= C / 4) on a GPU with C compute units: the workspace entry
+    point gives the first C rows a workgroup each and cuts the excess rows into quarters, a
+    workgroup each.  Same bits as one workgroup per row, twice in a row on one workspace."""
+    cus = ops.num_compute_units(DEV)
+    T = cus + extra
+    segs = ops.split_segments(T, H)
+    print(f"[case] mixed T={T} P={P} H={H} segments per excess row={segs}", flush=True)
+    assert segs == (2 if H == 4608 else 4)   # rows of 9 chunks on 3 waves are halved, not quartered
+    cfg, inp = make(P, T, H, seed=80 + extra)
+    want = run(inp, False, alias=P - 1)
+    for i in range(2):
+        got = run(inp, True, alias=P - 1)
+        assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]), f"call {i}"
+
+
+def test_mixed_launch_limits_and_oracle_parity(oracle):
+    cus = ops.num_compute_units(DEV)
+    assert ops.split_segments(cus, 8192) == 1                    # exactly one row per unit: nothing to balance
+    assert ops.split_segments(cus + cus // 4 + 1, 8192) == 1     # quarters would queue two deep on a unit
+    assert ops.split_segments(cus + 8, 8192, MAX_CTAS=64) == 1   # a grid cap is honoured by not cutting rows
+    assert ops.split_segments(cus + 8, 16384) == 1               # rows of more than 1024 vectors: other shape
+    assert ops.split_segments(cus + 8, 8200) == 1
+    T = cus + 45
+    cfg, inp = make(8, T, 8192, seed=97)
+    y, r = run(inp, None)                                        # the default route of the public op
+    y_w, r_w = oracle.reduce_add_rms_norm([to_bits(p) for p in inp.partials], to_bits(inp.residual),
+                                          to_bits(inp.weight), cfg.eps)
+    assert_parity(y, r, y_w, r_w, f"mixed T={T}")
+
+
 def test_workspace_argument_checks():
     L = _lib.lib()
     cfg, inp = make(2, 4, 1024, seed=61)

@@ -336,7 +336,10 @@ def prepare_split_workspace(device=None, stream: Optional[torch.cuda.Stream] = N
 
 
 def _wants_split(T: int, cap: int) -> bool:
-    return cap <= 0 and 0 < T <= _lib.TW_SPLIT_MAX_TOKENS
+    """Whether an uncapped call of T rows goes through the workspace entry point: decode-size
+    batches (split rows) and batches of a few more rows than compute units (mixed launch); the
+    library decides which kernel runs, the workspace is only made available here."""
+    return cap <= 0 and 0 < T <= 2 * _lib.TW_SPLIT_MAX_TOKENS
 
 
 def _fused_rs_ln(entry: str, kname: str, input, residual, weight, mcptr, signal_pads, rank,

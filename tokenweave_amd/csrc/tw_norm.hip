@@ -613,58 +613,74 @@ __device__ __forceinline__ void store16_device(__amdgpu_buffer_rsrc_t d, uint32_
   __builtin_amdgcn_raw_buffer_store_b128(t, d, off, 0, kStoreDevice);
 }
 
-template <int NP, bool XCD_ROWS>
-__global__ __launch_bounds__(1024) void row_norm_split_kernel(
-    PartialPtrs parts, int np_rt, void* y_out, void* residual, const void* __restrict__ weight,
-    SplitRow* __restrict__ ws, float eps, int num_tokens, int vec_per_row, float hidden, int segs, int nt) {
-  __shared__ uint32_t arrivals_before;
-  // nt = lanes per workgroup, as a kernel argument (see row_norm_vec_body)
+// One segment of a split row: VPT * nwaves whole chunks starting at chunk `chunk0` of row
+// `row` (wave w of the workgroup owns chunks chunk0 + k * nwaves + w, k < VPT: the same
+// lane-to-vector assignment as the row kernel's, segment by segment).  `lds_flag` is one
+// LDS word of the caller's.
+template <int NP, int VPT>
+__device__ __forceinline__ void split_segment(
+    const PartialPtrs& parts, int np_rt, void* y_out, void* residual, const void* __restrict__ weight,
+    SplitRow* __restrict__ slot, float eps, int row, int chunk0, int vec_per_row, float hidden, int segs, int nt,
+    uint32_t* lds_flag) {
   const int nwaves = nt >> 6;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int nchunks = (vec_per_row + 63) >> 6;
   const int np = NP > 0 ? NP : np_rt;
   const uint32_t row_bytes = (uint32_t)vec_per_row * 16u;
-
-  const int per_group = 8 * segs;
-  const int row = XCD_ROWS ? (blockIdx.x / per_group) * 8 + (blockIdx.x & 7) : blockIdx.x / segs;
-  const int seg = XCD_ROWS ? (blockIdx.x % per_group) >> 3 : blockIdx.x % segs;
-  // The first partial's pointer is demanded here so that its load goes out with the
-  // row count's: one round trip to the kernel arguments ahead of the test, and the loads
-  // that follow find their cache lines there.
-  asm volatile("" ::"s"(parts.p[0]));
-  if (row >= num_tokens) return;
-  const int chunk = seg * nwaves + wave;  // this wave's chunk of the row
-  const uint32_t off = (uint32_t)(chunk * 64 + lane) * 16u;
+  uint32_t off[VPT];
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) off[k] = (uint32_t)((chunk0 + k * nwaves + wave) * 64 + lane) * 16u;
 
   const __amdgpu_buffer_rsrc_t dr = row_desc(residual, row, row_bytes);
-  float s[8];
+  float s[VPT][8];
   if (NP > 0) {
-    uint4 a[NP > 0 ? NP : 1];
+    uint4 a[VPT][NP > 0 ? NP : 1];
+    uint4 rv[VPT];
 #pragma unroll
-    for (int p = 0; p < NP; ++p) a[p] = load16<kLoadStream>(row_desc(parts.p[p], row, row_bytes), off);
-    const uint4 rv = load16<kLoadStream>(dr, off);
-    unpack8(a[0], s);
+    for (int p = 0; p < NP; ++p) {
+      const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[p], row, row_bytes);
 #pragma unroll
-    for (int p = 1; p < NP; ++p) add8(a[p], s);
-    add8(rv, s);
+      for (int k = 0; k < VPT; ++k) a[k][p] = load16<kLoadStream>(dp, off[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) rv[k] = load16<kLoadStream>(dr, off[k]);
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) unpack8(a[k][0], s[k]);
+#pragma unroll
+    for (int p = 1; p < NP; ++p) {
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) add8(a[k][p], s[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) add8(rv[k], s[k]);
   } else {
-    unpack8(load16<kLoadStream>(row_desc(parts.p[0], row, row_bytes), off), s);
-    for (int p = 1; p < np; ++p) add8(load16<kLoadStream>(row_desc(parts.p[p], row, row_bytes), off), s);
-    add8(load16<kLoadStream>(dr, off), s);
+    {
+      const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[0], row, row_bytes);
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) unpack8(load16<kLoadStream>(dp, off[k]), s[k]);
+    }
+    for (int p = 1; p < np; ++p) {
+      const __amdgpu_buffer_rsrc_t dp = row_desc(parts.p[p], row, row_bytes);
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dp, off[k]), s[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) add8(load16<kLoadStream>(dr, off[k]), s[k]);
   }
 
-  SplitRow* slot = ws + row;
-  {
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
     float ss = 0.0f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) ss += s[e] * s[e];
+    for (int e = 0; e < 8; ++e) ss += s[k][e] * s[k][e];
     uint4 rnew;
-    rnew.x = pack_bf16(s[0], s[1]);
-    rnew.y = pack_bf16(s[2], s[3]);
-    rnew.z = pack_bf16(s[4], s[5]);
-    rnew.w = pack_bf16(s[6], s[7]);
-    store16_device(dr, off, rnew);
+    rnew.x = pack_bf16(s[k][0], s[k][1]);
+    rnew.y = pack_bf16(s[k][2], s[k][3]);
+    rnew.z = pack_bf16(s[k][4], s[k][5]);
+    rnew.w = pack_bf16(s[k][6], s[k][7]);
+    store16_device(dr, off[k], rnew);
     const float c = wave_sum(ss);
+    const int chunk = chunk0 + k * nwaves + wave;
     if (lane == 0 && chunk < nchunks)
       __hip_atomic_store(&slot->sums[chunk], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -695,9 +711,9 @@ __global__ __launch_bounds__(1024) void row_norm_split_kernel(
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (threadIdx.x == 0)
-    arrivals_before = __hip_atomic_fetch_add(&slot->arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *lds_flag = __hip_atomic_fetch_add(&slot->arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
-  if (arrivals_before != (uint32_t)(segs - 1)) return;
+  if (*lds_flag != (uint32_t)(segs - 1)) return;
 
   // Last workgroup of the row: all chunk sums are in the slot.
   if (threadIdx.x == 0) __hip_atomic_store(&slot->arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -730,6 +746,63 @@ __global__ __launch_bounds__(1024) void row_norm_split_kernel(
       store16(dy, (uint32_t)(v0 + u * nt) * 16u, o);
     }
   }
+}
+
+template <int NP, bool XCD_ROWS>
+__global__ __launch_bounds__(1024) void row_norm_split_kernel(
+    PartialPtrs parts, int np_rt, void* y_out, void* residual, const void* __restrict__ weight,
+    SplitRow* __restrict__ ws, float eps, int num_tokens, int vec_per_row, float hidden, int segs, int nt) {
+  __shared__ uint32_t arrivals_before;
+  // nt = lanes per workgroup, as a kernel argument (see row_norm_vec_body)
+  const int per_group = 8 * segs;
+  const int row = XCD_ROWS ? (blockIdx.x / per_group) * 8 + (blockIdx.x & 7) : blockIdx.x / segs;
+  const int seg = XCD_ROWS ? (blockIdx.x % per_group) >> 3 : blockIdx.x % segs;
+  // The first partial's pointer is demanded here so that its load goes out with the
+  // row count's: one round trip to the kernel arguments ahead of the test, and the loads
+  // that follow find their cache lines there.
+  asm volatile("" ::"s"(parts.p[0]));
+  if (row >= num_tokens) return;
+  split_segment<NP, 1>(parts, np_rt, y_out, residual, weight, ws + row, eps, row, seg * (nt >> 6), vec_per_row,
+                       hidden, segs, nt, &arrivals_before);
+}
+
+// ---------------------------------------------------------------------------
+// Mixed launch: a few more rows than compute units.
+//
+// With one workgroup per row, row counts just above the number of compute units leave
+// some units with two rows and the rest with one, and the launch takes as long as two
+// rows on one unit: 257 .. 400 rows all cost what 512 do.  Here the first `full` rows (one
+// per compute unit) go to one workgroup each as usual, and the excess rows are cut into
+// `segs` segments (halves or quarters of a row), each a workgroup of its own, handed over
+// through the workspace like the split rows above: every unit then carries its row plus
+// at most one segment (the launcher offers this up to a quarter more rows than units).  Same
+// bits as the one-workgroup kernel (the chunk sums are reduced
+// in the same order).  Workgroup b >= full serves excess row 8 ((b - full) / (8 segs)) +
+// b % 8, segment ((b - full) / 8) % segs (`full` is a multiple of 8: the segments of a row
+// share an XCD).
+// ---------------------------------------------------------------------------
+template <int NP, int SEG_VPT>
+__global__ __launch_bounds__(256) void row_norm_mixed_kernel(
+    PartialPtrs parts, int np_rt, void* y_out, void* residual, const void* __restrict__ weight,
+    SplitRow* __restrict__ ws, float eps, int num_tokens, int vec_per_row, float hidden, int full, int segs,
+    int nt) {
+  __shared__ float slots[2][kMaxChunks];
+  __shared__ float max_slots[2][16];
+  __shared__ uint32_t arrivals_before;
+  if ((int)blockIdx.x < full) {
+    // rows [0, full): exactly one row per workgroup (row loop with stride = row count)
+    row_norm_vec_body<__bf16, NP, 4, 256, true, false, kQNone>(parts, np_rt, y_out, residual, nullptr, weight,
+                                                              nullptr, nullptr, eps, full, vec_per_row, hidden, nt,
+                                                              full, slots, max_slots);
+    return;
+  }
+  const int b = (int)blockIdx.x - full;
+  const int per_group = 8 * segs;
+  const int row = full + (b / per_group) * 8 + (b & 7);
+  const int seg = (b % per_group) >> 3;
+  if (row >= num_tokens) return;
+  split_segment<NP, SEG_VPT>(parts, np_rt, y_out, residual, weight, ws + (row - full), eps, row,
+                             seg * SEG_VPT * (nt >> 6), vec_per_row, hidden, segs, nt, &arrivals_before);
 }
 
 // ---------------------------------------------------------------------------
@@ -989,6 +1062,56 @@ static void launch_split(const RowNormArgs& a, const SplitPlan& sp) {
                 a.split_ws, a.eps, (int)a.T, V, (float)a.H, sp.segs, sp.nwaves * 64);
 }
 
+// Mixed launch (row_norm_mixed_kernel) for cus < T <= cus + cus / 4 rows of at most 1024
+// vectors: `full` = cus rows with a workgroup each, the T - cus excess rows in quarters (halves
+// for rows too short to quarter), so that no compute unit gets more than one segment beside
+// its row.  Measured at hidden size 8192, eight partials, cold operands, 256 compute units:
+// 257 / 288 / 320 rows 11.0 / 11.8 / 12.1 us against 12.3 / 13.3 / 13.0 us with one workgroup
+// per row.  Beyond cus / 4 excess rows it stops paying: quarters then queue two deep on a unit
+// (321 rows 12.5 against 13.0 us, 352 rows 13.5 against 13.1, 376 rows 14.3 against 13.4), and
+// halves — one per unit up to cus / 2 excess rows — lose from the start (376 rows 14.0 against
+// 13.4 us): the workgroup that arrives last re-reads and normalises the whole row, which puts
+// nearly a second row's traffic back on its unit.  The workgroup shape is the row kernel's for
+// these sizes: four vectors per lane.
+struct MixedPlan { int full, segs, nt; };
+
+static bool mixed_plan(int V, int64_t T, int np, int cus, MixedPlan* mp) {
+  if (cus < 8 || cus % 8 != 0 || T <= cus || T > cus + cus / 4 || T - cus > TW_SPLIT_MAX_TOKENS) return false;
+  VecShape sh;
+  if (!vec_shape(V, T, np, &sh) || sh.vpt != 4 || sh.maxnt != 256) return false;
+  const int nwaves = sh.nt / 64;
+  const int nchunks = (V + 63) / 64;
+  if (nchunks < 2 * nwaves) return false;  // a half row must be whole chunks of its own
+  mp->full = cus;
+  mp->segs = nchunks > 3 * nwaves ? 4 : 2;
+  mp->nt = sh.nt;
+  return true;
+}
+
+template <int NP>
+static void launch_mixed(const RowNormArgs& a, const MixedPlan& mp) {
+  const int V = (int)(a.H / 8);
+  const int excess = (int)a.T - mp.full;
+  const int groups = (excess + 7) / 8;
+  dim3 g((unsigned)(mp.full + groups * 8 * mp.segs)), b((unsigned)mp.nt);
+#define TW_LAUNCH_MIXED(SEG_VPT)                                                                             \
+  launch_kernel(row_norm_mixed_kernel<NP, SEG_VPT>, g, b, 0, a.stream, a.parts, a.np, a.y, a.residual,       \
+                a.weight, a.split_ws, a.eps, (int)a.T, V, (float)a.H, mp.full, mp.segs, mp.nt)
+  if (mp.segs == 4) TW_LAUNCH_MIXED(1);
+  else TW_LAUNCH_MIXED(2);
+#undef TW_LAUNCH_MIXED
+}
+
+static void launch_mixed_np(const RowNormArgs& a, const MixedPlan& mp) {
+  switch (a.np) {
+    case 1: launch_mixed<1>(a, mp); break;
+    case 2: launch_mixed<2>(a, mp); break;
+    case 4: launch_mixed<4>(a, mp); break;
+    case 8: launch_mixed<8>(a, mp); break;
+    default: launch_mixed<0>(a, mp); break;
+  }
+}
+
 static void launch_split_np(const RowNormArgs& a, const SplitPlan& sp) {
   switch (a.np) {
     case 1: launch_split<1>(a, sp); break;
@@ -1119,9 +1242,15 @@ static int run_row_norm_any(const char* what, const void* const* partials, int n
   // budget and is honoured by not splitting.
   if (split_workspace && max_ctas <= 0 && splittable(vec_ok, dtype, residual, copy_out, quant)) {
     SplitPlan sp;
+    MixedPlan mp;
     if (split_plan((int)(H / 8), T, device_compute_units(), &sp)) {
       a.split_ws = static_cast<SplitRow*>(split_workspace);
       launch_split_np(a, sp);
+      return finish_launch(what);
+    }
+    if (mixed_plan((int)(H / 8), T, np, device_compute_units(), &mp)) {
+      a.split_ws = static_cast<SplitRow*>(split_workspace);
+      launch_mixed_np(a, mp);
       return finish_launch(what);
     }
   }
@@ -1209,8 +1338,11 @@ int run_row_norm_noalloc(const char* what, const void* const* partials, int np, 
 
 int split_segments(int64_t T, int64_t H, int max_ctas) {
   SplitPlan sp;
+  MixedPlan mp;
   if (max_ctas > 0 || H <= 0 || H % 8 != 0 || H / 8 > INT32_MAX) return 1;
-  return split_plan((int)(H / 8), T, device_compute_units(), &sp) ? sp.segs : 1;
+  if (split_plan((int)(H / 8), T, device_compute_units(), &sp)) return sp.segs;
+  // (the mixed plan's shape does not depend on the number of partials for these row counts)
+  return mixed_plan((int)(H / 8), T, 8, device_compute_units(), &mp) ? mp.segs : 1;
 }
 
 int run_row_norm(const char* what, const void* const* partials, int np, void* y,

@@ -253,8 +253,9 @@ void fused_rs_ln(bool all_gather, const char* kernel, Tensor& input, Tensor& res
   TORCH_CHECK(rank >= 0 && rank < world_size, "Invalid rank ", rank, ", must be in [0, ", world_size - 1, "]");
   const int64_t stride = peer_stride((uint64_t)mcptr, world_size, r.T * r.H * 2);
   Launch l(input);
-  if (max_ctas <= 0 && r.T > 0 && r.T <= TW_SPLIT_MAX_TOKENS) {
-    // decode-size batch: several workgroups per row where that pays
+  if (max_ctas <= 0 && r.T > 0 && r.T <= 2 * TW_SPLIT_MAX_TOKENS) {
+    // decode-size batch, or a few more rows than compute units: the workspace entry point
+    // cuts rows into several workgroups where that pays
     if (void* ws = split_workspace(dev, l.stream)) {
       check_rc(tw_fused_rs_ln_ag_cta_ws(input.data_ptr(), residual.data_ptr(), weight.data_ptr(), (uint64_t)mcptr,
                                         stride, (int)rank, (int)world_size, 0, (float)epsilon, r.T, r.H, ws,

@@ -402,3 +402,27 @@ def test_tuner_returns_a_well_formed_table():
     assert any("split_offset=" in ln for ln in lines)
     plan = tw.weave_plan(1024, {1024: e})
     assert plan is None or plan["split_size"] == tw.tokenweave_split_size(1024, e["split_offset"])
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 384, 72), (300, 384, 200), (645, 520, 136), (2458, 8192, 3696),
+                                   (1024, 8192, 7392), (333, 256, 1000), (2048, 10240, 328)])
+def test_gemm_inner_dimension_not_a_multiple_of_the_slab(M, N, K):
+    """K % 64 != 0 on the large-tile kernel (Qwen2's row-parallel MLP slices are 3696 and
+    7392 wide): the last k-slab's chunks past K are zero-filled.  Against fp32 CPU arithmetic,
+    and BIT-identical to the same product with both operands zero-padded to a whole number
+    of slabs (the padded columns add exact zeros in the same k-steps)."""
+    print(f"[case] gemm K tail M={M} N={N} K={K}", flush=True)
+    g = wl.make_gemm_inputs(M, N, K, DEV, seed=M + N + K)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16_nt(out, g.a, g.b)
+    Kp = (K + 63) // 64 * 64
+    ap = torch.zeros((M, Kp), dtype=torch.bfloat16, device=DEV)
+    bp = torch.zeros((N, Kp), dtype=torch.bfloat16, device=DEV)
+    ap[:, :K] = g.a
+    bp[:, :K] = g.b
+    padded = torch.empty_like(out)
+    ops.gemm_bf16_nt(padded, ap, bp)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), padded.view(torch.int16)), "differs from the zero-padded product"
+    if M * N * K <= 2458 * 8192 * 3696:
+        check(out, g.a, g.b, f"K tail {M}x{N}x{K}")

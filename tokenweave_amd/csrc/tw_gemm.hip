@@ -12,7 +12,7 @@
 // whole 128-byte lines per row.
 //
 // Two kernels:
-//  * gemm_bf16_nt_big_kernel<TM, TN> (K % 64 == 0): (64 TM) x (128 TN) x 64 tiles,
+//  * gemm_bf16_nt_big_kernel<TM, TN> (K >= 64; a last partial k-slab is zero-filled): (64 TM) x (128 TN) x 64 tiles,
 //    8 waves (2 x 4, two per SIMD), each wave (32 TM) x (32 TN): 128/192/256/320 x 256
 //    (TN = 2) chosen per problem so that the tile count wastes the fewest workgroup
 //    rounds (M = 2458: 320-row tiles make exactly 256 tiles; M = 1024: 128-row tiles
@@ -221,6 +221,32 @@ __device__ __forceinline__ void big_issue_slab(__amdgpu_buffer_rsrc_t da, __amdg
     __builtin_amdgcn_raw_ptr_buffer_load_lds(db, (lds_void_t*)(sb + j * 1024), 16, vb[j], koff, 0, 0);
 }
 
+// The last k-slab of an inner dimension that is not a multiple of 64 (but of 8): the 16-byte
+// chunks that lie past K must land in LDS as zeros.  A lane's chunk is c ^ 4 in odd 8-row
+// blocks and c in even ones (the swizzle above), so two flags per lane say whether its chunk
+// is inside; a chunk outside is requested at an offset past the descriptor's extent, which
+// the hardware answers with zeros.
+constexpr uint32_t BIG_OUT_OF_RANGE = 0x80000000u;  // operands are smaller than 2 GiB
+
+template <int LA, int LB>
+__device__ __forceinline__ void big_issue_slab_tail(__amdgpu_buffer_rsrc_t da, __amdgpu_buffer_rsrc_t db,
+                                                    const uint32_t (&va)[LA], const uint32_t (&vb)[LB],
+                                                    uint8_t* sa, uint8_t* sb, uint32_t koff, int blk_a, int blk_b,
+                                                    bool in_even, bool in_odd) {
+#pragma unroll
+  for (int j = 0; j < LA; ++j) {
+    const bool in = ((blk_a + j) & 1) ? in_odd : in_even;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(da, (lds_void_t*)(sa + j * 1024), 16, in ? va[j] : BIG_OUT_OF_RANGE, koff,
+                                             0, 0);
+  }
+#pragma unroll
+  for (int j = 0; j < LB; ++j) {
+    const bool in = ((blk_b + j) & 1) ? in_odd : in_even;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(db, (lds_void_t*)(sb + j * 1024), 16, in ? vb[j] : BIG_OUT_OF_RANGE, koff,
+                                             0, 0);
+  }
+}
+
 // `count` independent products of one shape in one launch: out[p] = a[p] * b[p]^T.  The
 // token-weave producer uses it for the P row-parallel partial sums of a token split,
 // each written into its rank's staging slot; a plain GEMM is count = 1.
@@ -247,12 +273,15 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
   const int wm = wave >> 2, wn = wave & 3, l32 = lane & 31, lhi = lane >> 5;
   const int tiles_per_product = tiles_m * tiles_n;
   const int num_tiles = count * tiles_per_product;
-  const int nk = K / BIG_BK;
+  const int nk = (K + BIG_BK - 1) / BIG_BK;
+  const int tail_chunks = (K % BIG_BK) / 8;  // 16-byte chunks of the last slab that lie inside K (0: all eight)
   // Loader: wave instruction j of wave w fills the 8-row LDS block w * L + j; lane l
   // lands at row l / 8, position l % 8 of that block, so it must fetch the chunk
   // (l % 8) ^ key(row), key(r) = (r >> 1) & 7 = ((block & 1) << 2) | (l >> 4).
   const int ld_row = lane >> 3;
   const int ld_key = lane >> 4;
+  const bool tail_in_even = ((lane & 7) ^ ld_key) < tail_chunks;
+  const bool tail_in_odd = ((lane & 7) ^ ld_key ^ 4) < tail_chunks;
   // Reader: lane row l32 (+ 32 i; wave offsets are multiples of 16 rows, which do not
   // change the key), chunk 2 kk + lhi.
   uint32_t roff[4];
@@ -314,10 +343,14 @@ __global__ __launch_bounds__(BIG_THREADS) void gemm_bf16_nt_big_kernel(
 
     for (int kt = 0; kt < nk; ++kt) {
       const int stage = kt & 1;
-      if (kt + 1 < nk)
+      if (kt + 2 < nk || (kt + 2 == nk && tail_chunks == 0))
         big_issue_slab<LA, LB>(da, db, va, vb, lds_big + (stage ^ 1) * STAGE + (wave * LA) * 1024,
                                lds_big + (stage ^ 1) * STAGE + PANEL_A + (wave * LB) * 1024,
                                (uint32_t)(kt + 1) * BIG_ROWB);
+      else if (kt + 2 == nk)
+        big_issue_slab_tail<LA, LB>(da, db, va, vb, lds_big + (stage ^ 1) * STAGE + (wave * LA) * 1024,
+                                    lds_big + (stage ^ 1) * STAGE + PANEL_A + (wave * LB) * 1024,
+                                    (uint32_t)(kt + 1) * BIG_ROWB, wave * LA, wave * LB, tail_in_even, tail_in_odd);
       const uint8_t* pa = lds_big + stage * STAGE + (wm * WM) * BIG_ROWB;
       const uint8_t* pb = lds_big + stage * STAGE + PANEL_A + (wn * WN) * BIG_ROWB;
       if constexpr (TN == 3) {
@@ -554,10 +587,11 @@ static BigTile pick_big_tile(int64_t M, int64_t N, int count, int cus) {
 // The tile shape never changes a result bit: every output element is the same sequence of
 // MFMA k-steps whatever tile it lies in.
 static bool big_kernel_fits(int64_t M, int64_t N, int64_t K) {
-  // whole 64-wide k-slabs, 32-bit byte offsets into both operands, and enough rows and
+  // at least one whole 64-wide k-slab, 32-bit byte offsets into both operands (below the
+  // out-of-range marker when a last partial slab has to be zero-filled), and enough rows and
   // columns to be worth the larger prologue
-  return (K % BIG_BK == 0) && ((uint64_t)M * K < (1ull << 31)) && ((uint64_t)N * K < (1ull << 31)) && M >= 192 &&
-         N >= 192;
+  const uint64_t limit = (K % BIG_BK == 0) ? (1ull << 31) : (1ull << 30);  // elements per operand
+  return K >= BIG_BK && (uint64_t)M * K < limit && (uint64_t)N * K < limit && M >= 192 && N >= 192;
 }
 
 static int launch_big_for(const GemmBatch& batch, int count, int64_t M, int64_t N, int64_t K, int64_t ldc,

@@ -212,8 +212,33 @@ REGIONS = 21        # timed regions of exactly `steps` launches each; the median
 LEAD_IN = 40        # untimed launches ahead of an event bracket (the bracket starts in a busy queue)
 
 
+def graph_replay_us(runner, launches, replays=5, brackets=7):
+    """`launches` consecutive steps of `runner` captured into one HIP graph, replayed `replays`
+    times per HIP-event bracket: microseconds per launch, median / min / max of `brackets`."""
+    import torch
+    main_s, _ = weave_streams()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=main_s):
+        for i in range(launches):
+            runner.step(i, main_s)
+    ts = []
+    with torch.cuda.stream(main_s):
+        g.replay()
+        torch.cuda.synchronize()
+        for _ in range(brackets):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(main_s)
+            for _ in range(replays):
+                g.replay()
+            e1.record(main_s)
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3 / (replays * launches))
+    del g
+    return statistics.median(ts), min(ts), max(ts)
+
+
 def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16", regions=REGIONS, preroll_ms=PREROLL_MS,
-              lead_in=LEAD_IN, split=None, pretouch=0):
+              lead_in=LEAD_IN, split=None, pretouch=0, graph=False):
     """After an untimed pre-roll and `warmup` warm-up launches, times `regions` regions of
     exactly `steps` back-to-back launches twice over: by the wall clock between two device
     synchronisations (ms_per_step, gbps), and by HIP events on the launch stream around
@@ -268,6 +293,9 @@ def time_norm(cfg, steps, warmup, max_ctas, device, epilogue="bf16", regions=REG
            "event_us_per_launch_min": min(events) * 1e6 / steps,
            "event_us_per_launch_max": max(events) * 1e6 / steps,
            "regions": regions, "preroll_steps": preroll_steps, "lead_in_steps": lead_in}
+    if graph:
+        # (c) the same launches with no host in the loop: two passes over the input sets in one graph
+        res["graph_replay_us_per_launch"], _, _ = graph_replay_us(runner, 2 * nsets)
     del runner
     torch.cuda.empty_cache()
     return res
@@ -326,28 +354,11 @@ def time_graph_replay(cfg, max_ctas, device, cycles=2, replays=5, brackets=7):
     import torch
     nsets = max(2, min(256, -(-ROTATION_BYTES // cfg.bytes)))
     runner = NormRunner(cfg, nsets, max_ctas, device)
-    main_s, _ = weave_streams()
-    launches = cycles * nsets
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g, stream=main_s):
-        for i in range(launches):
-            runner.step(i, main_s)
-    ts = []
-    with torch.cuda.stream(main_s):
-        g.replay()
-        torch.cuda.synchronize()
-        for _ in range(brackets):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(main_s)
-            for _ in range(replays):
-                g.replay()
-            e1.record(main_s)
-            torch.cuda.synchronize()
-            ts.append(e0.elapsed_time(e1) * 1e3 / (replays * launches))
-    out = {"workload": cfg.name, "launches_per_graph": launches, "rotating_input_sets": nsets,
+    med, lo, hi = graph_replay_us(runner, cycles * nsets, replays, brackets)
+    out = {"workload": cfg.name, "launches_per_graph": cycles * nsets, "rotating_input_sets": nsets,
            "replays_per_bracket": replays, "brackets": brackets,
-           "us_per_launch": round(statistics.median(ts), 3), "min": round(min(ts), 3), "max": round(max(ts), 3)}
-    del g, runner
+           "us_per_launch": round(med, 3), "min": round(lo, 3), "max": round(hi, 3)}
+    del runner
     torch.cuda.empty_cache()
     return out
 
@@ -1074,7 +1085,8 @@ def main():
     log(f"[bench] {torch.cuda.get_device_name(0)}; workload {cfg.name}: P={cfg.P} T={cfg.T} "
         f"H={cfg.H} bytes/call={cfg.bytes}")
 
-    res = time_norm(cfg, args.steps, args.warmup, args.max_ctas, device, pretouch=args.pretouch)
+    res = time_norm(cfg, args.steps, args.warmup, args.max_ctas, device, pretouch=args.pretouch,
+                    graph=not args.pretouch)
     log(f"[bench] {res}")
     kernel_us = res["event_us_per_launch"]
     traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name, (None, None)) if args.max_ctas == 0 else (None, None)
@@ -1100,6 +1112,8 @@ def main():
                                         "included), median region",
                      "lead_in_steps": res["lead_in_steps"],
                      "event_us_per_launch": round(kernel_us, 3),
+                     "graph_replay_us_per_launch": (round(res["graph_replay_us_per_launch"], 3)
+                                                    if "graph_replay_us_per_launch" in res else None),
                      "event_us_per_launch_min_max": [round(res["event_us_per_launch_min"], 3),
                                                      round(res["event_us_per_launch_max"], 3)]},
     }

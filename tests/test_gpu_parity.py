@@ -527,3 +527,52 @@ def test_special_values_match_the_checker(oracle):
     yw = bits_to_f32(y_want)
     assert np.isnan(yw[0, 3]) and not np.isnan(yw[0, 4]) and np.isnan(yw[2]).all()   # inf * 0; NaN mean
     assert (bits_to_f32(y_want)[4] != 0).any(), "subnormal row was flushed by the checker?"
+
+
+# ---------------------------------------------------------------------------
+# The reference's own check of its TokenWeave kernels (they have no pytest): the
+# correctness gate inside the artifact microbenchmark, artifact/figure_4_10/bench.py:80-99
+# (inputs), :182-199 (oracle and comparison), :243-244 (tolerance), :270-271 (grid).
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("ctas", [2, 8, 64, 0])
+@pytest.mark.parametrize("bl", [64, 256, 2048, 4096])
+def test_artifact_microbenchmark_correctness_gate(bl, ctas):
+    """Per rank p of 8: staging rows U(-1, 1) * (p + 1) / (3 * 8) in bf16; residual and weight
+    the all-reduced sums of such draws.  Expected = all-reduce of the staging rows, then the
+    stock `RMSNorm(hidden, residual)`; got = `fused_rs_ln_ag_cta` on every rank's row shard
+    with the artifact's grid (`ctas`, or the shard's row count for 0); compared on the hidden
+    states with torch.allclose(atol = rtol = 4e-2), as the artifact does — and the updated
+    residual at the same tolerance, which the artifact does not look at."""
+    ws, H, eps = 8, 8192, 1e-5
+    print(f"[case] artifact gate BL={bl} ctas={ctas}", flush=True)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(42 + bl)
+
+    def draw(shape, p):
+        return ((torch.rand(shape, generator=g, device=DEV) * 2 - 1).to(torch.bfloat16) * ((p + 1) / (3 * ws)))
+
+    buf = tw.PartialsBuffer(ws, bl, H, rank=0, device=DEV)
+    for p in range(ws):
+        buf.slot(p).copy_(draw((bl, H), p))
+    residual = sum(draw((bl, H), p).float() for p in range(ws)).to(torch.bfloat16)
+    weight = sum(draw((H,), p).float() for p in range(ws)).to(torch.bfloat16)
+    layer = tw.RMSNorm(H, eps=eps, dtype=torch.bfloat16).to(DEV)
+    layer.weight.data.copy_(weight)
+    # expected: all-reduce (bf16 result), then the stock layer on copies
+    ref_hidden = buf.storage.float().sum(dim=0).to(torch.bfloat16)
+    ref_residual = residual.clone()
+    layer(ref_hidden, ref_residual)
+    # got: the fused op, one call per rank's shard (one GPU plays the eight ranks in turn)
+    blpr = bl // ws
+    hidden = buf.hidden_states(bl)
+    for rank in range(ws):
+        start = rank * blpr
+        rows = hidden[start:start + blpr]
+        ops.fused_rs_ln_ag_cta(rows, residual[start:start + blpr], layer.weight.data,
+                               buf.multicast_ptr + buf.offset_of_row(start), buf.signal_pad_ptrs_dev, 0, ws,
+                               ctas if ctas else blpr, eps)
+        # (y lands on slot 0's rows, which is what `input` aliases for rank 0 of the buffer; the other
+        # slots' rows of this shard are consumed, not written)
+    torch.cuda.synchronize()
+    assert torch.allclose(ref_hidden, hidden, atol=4e-2, rtol=4e-2)
+    assert torch.allclose(ref_residual, residual, atol=4e-2, rtol=4e-2)

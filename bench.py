@@ -79,6 +79,7 @@ def bench_lib():
         L.twb_trace_reduce_add_rms_norm.argtypes = [ctypes.POINTER(vp), ci, vp, vp, vp, i64, i64, ci, f32, vp, vp]
         L.twb_gemm_loop.argtypes = [ci, ci, i64, vp, vp, vp, ci, vp]
         L.twb_lds_read_rate.argtypes = [ci, ci, ci, vp, vp, vp, ci, vp]
+        L.twb_gemm_bf16_nt_tile.argtypes = [vp, vp, vp, i64, i64, i64, i64, ci, ci, vp]
         L.twb_last_error.restype = ctypes.c_char_p
         _BENCH_LIB = L
     return _BENCH_LIB
@@ -109,6 +110,9 @@ def parse_args():
                          "compute units (K = 1024 and 8192) with the shader clock rocm-smi reports meanwhile")
     ap.add_argument("--weave-only", action="store_true",
                     help="time only the GEMM + norm weave of config 5 and print its figures (for profiling)")
+    ap.add_argument("--weave-power", action="store_true",
+                    help="run every leg of config 5's stage for seconds each and print its time next to the "
+                         "socket power, shader clock and memory-controller activity rocm-smi reports meanwhile")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="after the timed region, run the library's plain copy kernel on "
                          "buffers of known size (reference traffic for rocprofv3 --pmc runs)")
@@ -1024,6 +1028,129 @@ def time_gemm_scaling(device, seconds=2.0):
     return out
 
 
+def board_metrics():
+    """Socket power (W), shader clock (MHz) and memory-controller activity (%) as
+    `rocm-smi --showmetrics` reports them right now; {} where the tool or a field is missing."""
+    import re
+    import subprocess
+    out = {}
+    try:
+        txt = subprocess.run(["rocm-smi", "--showmetrics"], capture_output=True, text=True, timeout=10).stdout
+    except Exception:
+        return out
+    for key, name in (("current_socket_power (W):", "watts"), ("current_gfxclk (MHz):", "sclk_mhz"),
+                      ("average_umc_activity (%):", "umc_pct")):
+        m = re.search(re.escape(key) + r"\s*([0-9.]+)\s*$", txt, re.M)
+        if m:
+            out[name] = float(m.group(1))
+    return out
+
+
+def time_weave_power(device, seconds=2.5):
+    """What the board draws while each leg of config 5's stage runs back to back for `seconds`:
+    socket power, shader clock and memory-controller activity (medians of `rocm-smi
+    --showmetrics` samples during the leg), the stage time (HIP events), and their product,
+    the energy one stage takes.  Legs per form (one rank's GEMM / all eight partial sums):
+    GEMM alone, norm alone, both on one stream, the two-stream stage at the GEMM budgets
+    128 and 240 compute units; for one rank's GEMM also the big kernel forced to its 192 x 256
+    and 128 x 256 tiles (164 and 124 registers per lane: a norm workgroup fits beside two of
+    its waves on every SIMD) alone and beside the uncapped norm on the second stream."""
+    import threading
+    import torch
+    from tokenweave_amd import _custom_ops as ops
+    from tokenweave_amd import workloads as wl
+    BL = bench_lib()
+    cfg = wl.C5_NORM
+    inps = [wl.make_norm_inputs(cfg, device, seed_offset=i) for i in range(8)]
+    norms = [ops.bind_reduce_add_rms_norm(inp.partials, inp.partials[0], inp.residual, inp.weight, cfg.eps, None)
+             for inp in inps]
+    main_s, side_s = weave_streams()
+    idle = board_metrics()
+    out = {"definitions": "us = stage time by HIP events; watts / sclk_mhz / umc_pct = medians of rocm-smi "
+                          "--showmetrics samples (current_socket_power, current_gfxclk, average_umc_activity) "
+                          "while the leg runs for `seconds`; mJ = watts x us",
+           "seconds": seconds, "idle": idle}
+
+    def run_leg(fn):
+        for i in range(10):
+            fn(i)
+        torch.cuda.synchronize()
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            while not stop.is_set():
+                samples.append(board_metrics())
+                time.sleep(0.05)
+        th = threading.Thread(target=sampler)
+        th.start()
+        ts, t_end = [], time.perf_counter() + seconds
+        while time.perf_counter() < t_end:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(main_s)
+            for i in range(100):
+                fn(i)
+            e1.record(main_s)
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3 / 100)
+        stop.set()
+        th.join()
+        row = {"us": round(statistics.median(ts), 2)}
+        for k in ("watts", "sclk_mhz", "umc_pct"):
+            v = [x[k] for x in samples[2:] if k in x]
+            row[k] = round(statistics.median(v), 1) if v else None
+        row["mJ"] = round(row["watts"] * row["us"] * 1e-3, 1) if row["watts"] else None
+        return row
+
+    def norm(i, stream):
+        norms[i % 8](stream)
+
+    def two_streams(gemm):
+        def stage(i):
+            before = torch.cuda.Event()
+            before.record(main_s)
+            gemm(i, main_s)
+            side_s.wait_event(before)
+            norm(i, side_s)
+            main_s.wait_stream(side_s)
+        return stage
+
+    for form, P in (("one_partial", 1), ("eight_partials", 8)):
+        gs = wl.make_partials_gemm_inputs(P, device=device)
+        Ta, K = gs[0].a.shape
+        N = gs[0].b.shape[0]
+        R = 4
+        stages = [torch.zeros((P, Ta, N), dtype=torch.bfloat16, device=device) for _ in range(R)]
+
+        def bind(cap):
+            if P == 1:
+                return [ops.bind_gemm_bf16_nt(st[0], gs[0].a, gs[0].b, cap or None) for st in stages]
+            return [ops.bind_gemm_bf16_nt_partials([st[p] for p in range(P)], [g.a for g in gs],
+                                                   [g.b for g in gs], cap or None) for st in stages]
+        gemms = {cap: bind(cap) for cap in (0, 128, 240)}
+        legs = {"gemm": lambda i: gemms[0][i % R](main_s),
+                "norm": lambda i: norm(i, main_s),
+                "serial": lambda i: (gemms[0][i % R](main_s), norm(i, main_s))}
+        for cap in (128, 240):
+            legs[f"gemm/{cap}"] = (lambda c: lambda i: gemms[c][i % R](main_s))(cap)
+            legs[f"weave/{cap}"] = two_streams((lambda c: lambda i, s: gemms[c][i % R](s))(cap))
+        if P == 1:
+            for tm in (3, 2):
+                def forced(i, stream, tm=tm):
+                    bench_check(BL.twb_gemm_bf16_nt_tile(stages[i % R][0].data_ptr(), gs[0].a.data_ptr(),
+                                                         gs[0].b.data_ptr(), Ta, N, K, N, tm, 2,
+                                                         stream.cuda_stream))
+                legs[f"gemm_tile{64 * tm}x256"] = (lambda f: lambda i: f(i, main_s))(forced)
+                legs[f"same_units/tile{64 * tm}x256"] = two_streams(forced)
+        rows = {}
+        for name, fn in legs.items():
+            rows[name] = run_leg(fn)
+            log(f"[weave-power] {form} {name}: {rows[name]}")
+        out[form] = rows
+        del gemms, stages, gs
+        torch.cuda.empty_cache()
+    return out
+
+
 def weave_block(device, steps):
     """Both forms of config 5 for the JSON line."""
     caps = (128, 160, 176, 192, 208, 224, 240)
@@ -1081,6 +1208,9 @@ def main():
         return
     if args.weave_only:
         print(json.dumps({"weave": weave_block(device, 20)}), flush=True)
+        return
+    if args.weave_power:
+        print(json.dumps({"weave_power": time_weave_power(device)}), flush=True)
         return
     log(f"[bench] {torch.cuda.get_device_name(0)}; workload {cfg.name}: P={cfg.P} T={cfg.T} "
         f"H={cfg.H} bytes/call={cfg.bytes}")

@@ -537,6 +537,33 @@ TWB_API int twb_reduce_add_rms_norm_split_spread(const void* const* partials, in
   return tw::finish_launch(what);
 }
 
+// tw_gemm_bf16_nt with the big kernel's workgroup tile forced to (64 tm) x (128 tn), one
+// workgroup per tile and no compute-unit budget, instead of the tile the library's cost
+// model picks: the 192 x 256 and 128 x 256 tiles leave registers for a norm workgroup on
+// the same compute unit, which the 320 x 256 tile does not.  Same operand rules as the
+// library call; the shape must fit the big kernel.
+TWB_API int twb_gemm_bf16_nt_tile(void* out, const void* a, const void* b, int64_t M, int64_t N, int64_t K,
+                                  int64_t ldc, int tm, int tn, void* stream) {
+  const char* what = "gemm_bf16_nt_tile";
+  if (int rc = tw::check_gemm_shape(what, M, N, K, ldc)) return rc;
+  if (int rc = tw::check_gemm_pointers(what, out, a, b, nullptr)) return rc;
+  if (M == 0) return TW_OK;
+  if (!tw::big_kernel_fits(M, N, K)) return tw::set_error(TW_ERR_INVALID_ARGUMENT, "%s: shape outside the big kernel", what);
+  tw::GemmBatch batch = {};
+  batch.out[0] = static_cast<uint16_t*>(out);
+  batch.a[0] = static_cast<const uint16_t*>(a);
+  batch.b[0] = static_cast<const uint16_t*>(b);
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  int rc = TW_ERR_INVALID_ARGUMENT;
+  if (tm == 2 && tn == 2) rc = tw::launch_big<2, 2>(batch, 1, M, N, K, ldc, 0, hs);
+  else if (tm == 3 && tn == 2) rc = tw::launch_big<3, 2>(batch, 1, M, N, K, ldc, 0, hs);
+  else if (tm == 4 && tn == 2) rc = tw::launch_big<4, 2>(batch, 1, M, N, K, ldc, 0, hs);
+  else if (tm == 5 && tn == 2) rc = tw::launch_big<5, 2>(batch, 1, M, N, K, ldc, 0, hs);
+  else if (tm == 4 && tn == 3) rc = tw::launch_big<4, 3>(batch, 1, M, N, K, ldc, 0, hs);
+  else return tw::set_error(TW_ERR_INVALID_ARGUMENT, "%s: no %d x %d tile", what, 64 * tm, 128 * tn);
+  return rc ? rc : tw::finish_launch(what);
+}
+
 static int bench_lds_limit(const void* fn, int bytes) {
   return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess ? TW_OK
              : tw::set_error(TW_ERR_LAUNCH, "the device refused %d bytes of LDS", bytes);

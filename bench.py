@@ -932,6 +932,17 @@ def time_gemm_limits(device):
         loop[name] = {"cycles_per_slab": round(cyc / slabs), "mfma_issue_share": round(2560.0 * slabs / cyc, 3),
                       "shader_clock_ghz": round(cyc / wall_us / 1e3, 2), "tflops": round(flops / t / 1e12, 1),
                       "share_of_2.5_pflops": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 3)}
+        # socket power while the same launch repeats for two seconds
+        samples, t_end = [], time.perf_counter() + 2.0
+        while time.perf_counter() < t_end:
+            for _ in range(8):
+                bench_check(L.twb_gemm_loop(slabs, parts, window, src.data_ptr(), stamps.data_ptr(),
+                                            sink.data_ptr(), cus, sp))
+            samples.append(board_metrics())   # taken while the queued launches run
+            torch.cuda.synchronize()
+        watts = [x["watts"] for x in samples[2:] if "watts" in x]
+        loop[name]["socket_watts"] = round(statistics.median(watts)) if watts else None
+        log(f"[gemm-limits] {name}: {loop[name]}")
     lds = {}
     iters = 2000
     cyc_out = torch.zeros(cus, dtype=torch.int64, device=device)
